@@ -1,0 +1,48 @@
+"""ctypes binding of ``libhbsattn_amd.so`` (the C ABI in ``include/hbsattn_amd.h``)."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhbsattn_amd.so")
+ABI_VERSION = 1
+
+DTYPE_BF16 = 0
+DTYPE_F16 = 1
+
+_lib = None
+
+
+class HBSAttnLibraryError(RuntimeError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Open the built library.  There is no fallback: a missing or stale library is an error."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise HBSAttnLibraryError(
+            f"{LIB_PATH} is missing: build it with `python -m hbsattn_amd.build` (hipcc, gfx950). "
+            "hbsattn_amd has no fallback compute path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.hbsa_abi_version.restype = ctypes.c_int
+    lib.hbsa_abi_version.argtypes = []
+    if lib.hbsa_abi_version() != ABI_VERSION:
+        raise HBSAttnLibraryError(f"{LIB_PATH}: ABI version {lib.hbsa_abi_version()} != expected {ABI_VERSION}; rebuild")
+    lib.hbsa_last_error.restype = ctypes.c_char_p
+    lib.hbsa_last_error.argtypes = []
+    lib.hbsa_fwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.hbsa_fwd_workspace_bytes.argtypes = [ctypes.c_int32] * 3
+    vp = ctypes.c_void_p
+    lib.hbsa_fwd.restype = ctypes.c_int
+    lib.hbsa_fwd.argtypes = ([vp] * 11 + [ctypes.c_size_t] + [ctypes.c_int32] * 12 + [ctypes.c_float]
+                             + [ctypes.POINTER(ctypes.c_int64), vp])
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().hbsa_last_error().decode("utf-8", "replace")

@@ -1,0 +1,39 @@
+"""Builds ``libhbsattn_amd.so`` in-tree with hipcc for gfx950.
+
+``python -m hbsattn_amd.build`` or ``hbsattn_amd.build.build()``.  hipcc
+cross-compiles, so no GPU is needed to build.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_ROOT = os.path.dirname(_HERE)
+SOURCES = [os.path.join(_HERE, "csrc", "hbsa_fwd.hip")]
+OUTPUT = os.path.join(_HERE, "libhbsattn_amd.so")
+
+# -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-I" + os.path.join(_ROOT, "include"),
+]
+
+
+def build(verbose: bool = False) -> str:
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    cmd = [hipcc] + HIPCC_FLAGS + SOURCES + ["-o", OUTPUT]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+        raise RuntimeError("hipcc failed: " + " ".join(cmd))
+    if verbose:
+        print(" ".join(cmd))
+    return OUTPUT
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

@@ -1,0 +1,142 @@
+"""The public operator: same call as the reference's ``hbsattn.HBSAttention``.
+
+Mirrors reference ``hbsattn/hbsa_interface.py:6-35`` (a ``torch.autograd.Function``
+used through ``.apply``, positional arguments, no backward) and the host-side checks
+of its two launchers (reference ``hbsattn/fwd_triton_auto_tile_size.py:254-281``,
+``hbsattn/fwd_triton_fix_tile_size.py:216-242``).  Both ``tile_mode`` values run the
+one HIP kernel family; ``'fix'`` keeps the reference's power-of-two assertion so code
+that relies on it behaves the same.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .utils import calculate_blocks
+
+_NATIVE_HEADDIMS = (32, 64, 128)
+_DTYPE_CODES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16}
+
+
+def _as_int32(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype != torch.int32:
+        t = t.to(torch.int32)
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _rows_ok(t: torch.Tensor) -> bool:
+    """16-byte aligned rows with a unit head-dim stride are what the kernels load."""
+    return (t.stride(2) == 1 and t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0 and t.data_ptr() % 16 == 0)
+
+
+def _pad_headdim(t: torch.Tensor, d_pad: int) -> torch.Tensor:
+    out = t.new_zeros((t.shape[0], t.shape[1], d_pad))
+    out[:, :, : t.shape[2]] = t
+    return out
+
+
+def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, softmax_scale,
+                 num_q_block, q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block) -> torch.Tensor:
+    """Host launcher: checks, scratch allocation and one call through the C ABI.  No device
+    synchronisation happens here."""
+    if not q.is_cuda:
+        raise RuntimeError("hbsattn_amd runs on MI355X only: q/k/v must be CUDA(HIP) tensors; there is no CPU path")
+    if not (k.device == q.device and v.device == q.device and block_mask.device == q.device):
+        raise RuntimeError("q, k, v and block_mask must live on the same device")
+    if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
+        raise ValueError("q, k, v must have shape (total_tokens, nheads, headdim)")
+    if not (k.dtype == q.dtype and v.dtype == q.dtype):
+        raise TypeError("q, k and v must share one dtype")
+    if q.dtype not in _DTYPE_CODES:
+        raise TypeError(f"hbsattn_amd: dtype {q.dtype} is not supported (bfloat16 and float16 are)")
+    total_q, nhead_q, headdim = q.shape
+    total_k, nhead_k = k.shape[0], k.shape[1]
+    if k.shape[2] != headdim or v.shape != k.shape:
+        raise ValueError("k and v must have shape (total_k, nhead_k, headdim) with q's headdim")
+    assert nhead_q % nhead_k == 0, "nhead_q must be divisible by nhead_k (for GQA)"
+    assert q_block_size > 0 and k_block_size > 0 and q_block_size % 16 == 0 and k_block_size % 16 == 0, \
+        "q_block_size and k_block_size must be integer multiples of 16."
+    if headdim > _NATIVE_HEADDIMS[-1]:
+        raise NotImplementedError(f"hbsattn_amd: headdim {headdim} > {_NATIVE_HEADDIMS[-1]} is not supported")
+    scale = float(softmax_scale) if softmax_scale is not None else headdim ** -0.5
+
+    lib = _lib.load()
+    out = torch.empty((total_q, nhead_q, headdim), dtype=q.dtype, device=q.device)
+    if total_q == 0:
+        return out
+
+    d_run = next(d for d in _NATIVE_HEADDIMS if d >= headdim)
+    if d_run != headdim:  # zero columns add nothing to q.k and give zero output columns
+        q, k, v = _pad_headdim(q, d_run), _pad_headdim(k, d_run), _pad_headdim(v, d_run)
+        out_run = torch.empty((total_q, nhead_q, d_run), dtype=q.dtype, device=q.device)
+    else:
+        q = q if _rows_ok(q) else q.contiguous()
+        k = k if _rows_ok(k) else k.contiguous()
+        v = v if _rows_ok(v) else v.contiguous()
+        out_run = out
+
+    cu_q = _as_int32(cu_q_seqlens)
+    cu_k = _as_int32(cu_k_seqlens)
+    qb2b = _as_int32(q_block_to_batch)
+    cu_nqb = _as_int32(cu_num_q_block)
+    cu_nkb = _as_int32(cu_num_k_block)
+    batch = cu_q.numel() - 1
+
+    ws_bytes = int(lib.hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block))
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    strides = (ctypes.c_int64 * 11)(q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+                                    out_run.stride(0), out_run.stride(1), *block_mask.stride())
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.hbsa_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out_run.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),
+                          block_mask.data_ptr(), qb2b.data_ptr(), cu_nqb.data_ptr(), cu_nkb.data_ptr(),
+                          workspace.data_ptr(), ws_bytes, _DTYPE_CODES[q.dtype], batch, total_q, total_k, nhead_q,
+                          nhead_k, d_run, num_q_block, num_k_block, q_block_size, k_block_size, int(bool(causal)),
+                          scale, strides, stream)
+    if rc != 0:
+        raise RuntimeError(f"hbsa_fwd failed (code {rc}): {_lib.last_error()}")
+    # The launches are queued on `stream`; torch's caching allocator keeps `workspace` and any
+    # padded copies alive until work queued on that stream before their release has run.
+    if out_run is not out:
+        out.copy_(out_run[:, :, :headdim])
+    return out
+
+
+class _HBSAttentionFunction(torch.autograd.Function):
+    """Positional signature identical to reference ``hbsattn/hbsa_interface.py:9``."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal,
+                softmax_scale, tile_mode="auto", num_q_block=None, cu_q_block=None, q_block_to_batch=None,
+                cu_num_q_block=None, num_k_block=None, cu_k_block=None, k_block_to_batch=None, cu_num_k_block=None):
+        # Block metadata is all-or-recompute per side (reference hbsa_interface.py:14-17).
+        if num_q_block is None or cu_q_block is None or q_block_to_batch is None or cu_num_q_block is None:
+            num_q_block, cu_q_block, q_block_to_batch, cu_num_q_block = calculate_blocks(cu_q_seqlens, q_block_size)
+        if num_k_block is None or cu_k_block is None or k_block_to_batch is None or cu_num_k_block is None:
+            num_k_block, cu_k_block, k_block_to_batch, cu_num_k_block = calculate_blocks(cu_k_seqlens, k_block_size)
+
+        assert block_mask.dtype == torch.bool, "block_mask must be a boolean tensor"
+        assert block_mask.shape == (k.shape[1], num_q_block, num_k_block), (
+            "block_mask must be a boolean tensor of shape (nheads_k, num_q_block, num_k_block) = "
+            f"({k.shape[1]}, {num_q_block}, {num_k_block})")
+
+        if tile_mode == "auto":
+            pass
+        elif tile_mode == "fix":
+            assert (q_block_size & (q_block_size - 1) == 0) and (k_block_size & (k_block_size - 1) == 0), \
+                "q_block_size and k_block_size must be powers of 2"
+        else:
+            raise ValueError(f"Invalid tile mode: {tile_mode}")
+        return hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal,
+                            softmax_scale, int(num_q_block), q_block_to_batch, cu_num_q_block, int(num_k_block),
+                            cu_num_k_block)
+
+    @staticmethod
+    def backward(ctx, do):
+        raise NotImplementedError("It does not support gradient propagation yet")
+
+
+HBSAttention = _HBSAttentionFunction.apply

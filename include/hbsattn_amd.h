@@ -1,0 +1,95 @@
+/*
+ * C ABI of libhbsattn_amd.so — hand-written gfx950 (MI355X) kernels for the
+ * block-sparse attention forward that sits behind hbsattn.HBSAttention.
+ *
+ * The reference has no FFI for this path: its operator
+ * (reference hbsattn/hbsa_interface.py:9-27) calls a Python launcher that JIT-compiles
+ * a Triton kernel (reference hbsattn/fwd_triton_auto_tile_size.py:254-310 and
+ * hbsattn/fwd_triton_fix_tile_size.py:216-276).  The entry points below are what a
+ * binding for that launcher would need; each cites the reference code it replaces.
+ *
+ * Conventions
+ *   - every pointer named `*_dev` / tensor pointer is DEVICE memory owned by the
+ *     caller; the library never allocates, frees or retains device memory;
+ *   - all launches go to `stream` (a hipStream_t passed as void*; NULL = the null
+ *     stream) and the calls return without synchronising;
+ *   - return value 0 = success, negative = invalid argument (message available
+ *     through hbsa_last_error(), which is thread-local), positive = hipError_t;
+ *   - strides are in ELEMENTS; the innermost (head-dim) stride of q/k/v/out must be 1.
+ */
+#ifndef HBSATTN_AMD_H_
+#define HBSATTN_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HBSA_ABI_VERSION 1
+
+/* element types of q/k/v/out (reference: dtype follows the input tensors,
+ * hbsattn/fwd_triton_auto_tile_size.py:272) */
+#define HBSA_DTYPE_BF16 0
+#define HBSA_DTYPE_F16 1
+
+#define HBSA_ERR_INVALID_ARGUMENT (-1)
+#define HBSA_ERR_UNSUPPORTED (-2)
+#define HBSA_ERR_WORKSPACE_TOO_SMALL (-3)
+
+/* ABI version of the loaded library (== HBSA_ABI_VERSION it was built with). */
+int hbsa_abi_version(void);
+
+/* Message of the last failing call on this host thread ("" if none). */
+const char *hbsa_last_error(void);
+
+/*
+ * Bytes of device scratch hbsa_fwd needs for this problem.  Replaces the launcher's
+ * own scratch allocations (reference hbsattn/fwd_triton_auto_tile_size.py:273-274:
+ * `lse`, `tmp`); here the scratch holds the compacted work description the pre-pass
+ * builds (per-q-block geometry records and one bit per in-sequence k block).
+ * Depends only on host-known sizes, so no device synchronisation is needed.
+ */
+size_t hbsa_fwd_workspace_bytes(int32_t nhead_k, int32_t num_q_block, int32_t num_k_block);
+
+/*
+ * Block-sparse attention forward.  Replaces `_forward_auto_tile_size` and
+ * `_forward_fix_tile_size` + their Triton `_fwd_kernel`s (reference
+ * hbsattn/fwd_triton_auto_tile_size.py:76-310, hbsattn/fwd_triton_fix_tile_size.py:30-276).
+ *
+ *   q   [total_q, nhead_q, headdim]   k, v [total_k, nhead_k, headdim]   out like q
+ *   cu_q_seqlens, cu_k_seqlens  int32[batch+1]  packed-sequence boundaries
+ *   block_mask  bytes (0 / non-0) [nhead_k, num_q_block, num_k_block] over GLOBAL block
+ *               indices; entries pairing blocks of different sequences are ignored
+ *   q_block_to_batch int32[num_q_block], cu_num_q_block / cu_num_k_block int32[batch+1]
+ *               exactly as hbsattn.utils.calculate_blocks returns them
+ *               (reference hbsattn/utils.py:7-50)
+ *   causal      bottom-right aligned: in-sequence key j visible to in-sequence query i
+ *               iff i + (k_len - q_len) >= j
+ *   softmax_scale  already resolved (the caller substitutes headdim**-0.5 for None)
+ *   strides     int64[11] = { q_tok, q_head, k_tok, k_head, v_tok, v_head,
+ *                             out_tok, out_head, mask_head, mask_qblk, mask_kblk }
+ *   workspace   >= hbsa_fwd_workspace_bytes(...) bytes, 256-byte aligned
+ *
+ * Supported: headdim in {32, 64, 128}; q_block_size, k_block_size positive multiples
+ * of 16; nhead_q % nhead_k == 0; every sequence length >= 1.  Query rows with no
+ * visible key produce exactly 0 (reference hbsattn/reference.py:97-98).
+ */
+int hbsa_fwd(const void *q, const void *k, const void *v, void *out,
+             const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens,
+             const uint8_t *block_mask,
+             const int32_t *q_block_to_batch, const int32_t *cu_num_q_block,
+             const int32_t *cu_num_k_block,
+             void *workspace, size_t workspace_bytes,
+             int32_t dtype, int32_t batch, int32_t total_q, int32_t total_k,
+             int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+             int32_t num_q_block, int32_t num_k_block,
+             int32_t q_block_size, int32_t k_block_size,
+             int32_t causal, float softmax_scale,
+             const int64_t *strides, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HBSATTN_AMD_H_ */
