@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-sparse attention forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|T|C3|C4|C5]
+
+A step is one ``HBSAttention`` call (pre-pass + attention kernel, block metadata
+pre-computed and passed in as the reference's sweep does, reference
+test/test_speedup.py:101-102,152) on a synthetic problem already resident in HBM.  The
+timed region is ``synchronize -> K calls -> synchronize`` (reference hbsattn/benchmark.py:72-81
+brackets every call; the per-call figure measured that way is reported as
+``per_call_sync_ms``).  Prints ONE JSON line.
+
+``value`` is effective TFLOP/s over kept blocks: 4 * D * sum(rows(qb) * cols(kb)) over the
+visited block pairs of every q head, computed on the host from the mask, divided by the
+time of one step.  ``roofline`` prices the attention kernel alone (its launches are
+bracketed by events on the stream they are queued on); ``cpu_baseline`` times the CPU
+oracle (a port of the reference's golden implementation) on a bounded sample of the same
+workload on this machine's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, vendor figure
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, vendor figure
+
+DESCRIPTIONS = {
+    "C2": "C2: batch 8 x 8192 tokens, Hq=Hk=32, D=128, 128x128 blocks, keep 0.1 + diagonal, causal, bf16",
+    "T": "T: batch 8 x 32768 tokens, Hq=Hk=32, D=128, 128x128 blocks, keep 0.1 + diagonal, causal, bf16",
+    "C3": "C3: batch 8, lengths U[2048,16384], Hq=32 Hk=8, D=128, 64x128 blocks, keep 0.3 + diagonal, causal, bf16",
+    "C4": "C4: batch 8 x 65536 tokens, Hq=Hk=32, D=128, 128x128 blocks, keep 0.3, non-causal, bf16",
+    "C5": "C5: q lens 3000/5120/777/4096, k lens 6000/5120/4100/8192, Hq=16 Hk=2, D=64, 80x48 blocks, keep 0.5, causal, scale 0.1, bf16",
+}
+# which roof bounds the attention kernel at each workload (arithmetic intensity against the
+# ridge at 2500 TFLOP/s / 8 TB/s = 312 FLOP/B)
+BOUND = {"C2": "hbm", "T": "mfma", "C3": "mfma", "C4": "mfma", "C5": "hbm"}
+
+
+def time_steps(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
+def time_per_call_sync(fn, steps):
+    ts = []
+    for _ in range(steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        ts.append((time.perf_counter() - t0) * 1e3)
+    return sum(ts) / len(ts)
+
+
+def time_kernel_events(fn, steps):
+    """Average device time of ``fn``'s launches, from event pairs recorded on the current
+    stream (the stream the library launches on)."""
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in evs) / steps
+
+
+def measure(name, steps, warmup):
+    from hbsattn_amd import HBSAttention
+    from hbsattn_amd.interface import hbsa_prepare, hbsa_run
+    from hbsattn_amd.workloads import count_work, make_workload
+
+    w = make_workload(name, device="cuda", gen_device="device")
+    work = count_work(w)
+    args = w.args()
+    step = lambda: HBSAttention(*args)
+    ms = time_steps(step, steps, warmup)
+    per_call = time_per_call_sync(step, steps)
+    prepared = hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, w.q_block_size, w.k_block_size, w.causal,
+                            w.q_meta[0], w.q_meta[2], w.q_meta[3], w.k_meta[0], w.k_meta[3])
+    kernel_ms = time_kernel_events(lambda: hbsa_run(w.q, w.k, w.v, prepared, w.softmax_scale), steps)
+    prep_ms = time_kernel_events(
+        lambda: hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, w.q_block_size, w.k_block_size, w.causal,
+                             w.q_meta[0], w.q_meta[2], w.q_meta[3], w.k_meta[0], w.k_meta[3]), steps)
+    res = {
+        "ms_per_step": ms,
+        "per_call_sync_ms": per_call,
+        "attention_kernel_ms": kernel_ms,
+        "prepass_ms": prep_ms,
+        "tflops": work["flops"] / ms / 1e9,
+        "tflops_exact_elements": work["flops_exact"] / ms / 1e9,
+        "flops": work["flops"],
+        "bytes": work["bytes"],
+        "visited_pairs": work["visited_pairs"],
+    }
+    if BOUND[name] == "mfma":
+        ach = work["flops"] / kernel_ms / 1e9
+        res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                           "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "hbsa_fwd_kernel",
+                           "kernel_ms": kernel_ms, "algorithmic_flops": work["flops"]}
+    else:
+        ach = work["bytes"] / kernel_ms / 1e6
+        res["roofline"] = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                           "frac": ach / PEAK_HBM_GBS, "traffic": None, "kernel": "hbsa_fwd_kernel",
+                           "kernel_ms": kernel_ms, "algorithmic_bytes": work["bytes"],
+                           "mfma_frac": work["flops"] / kernel_ms / 1e9 / PEAK_BF16_TFLOPS}
+    return w, res
+
+
+def cpu_baseline(w, budget_s=20.0):
+    """The CPU oracle on sequence 0 of the workload, one kv head group at a time until the
+    budget is spent; throughput in the metric's unit from the sample's own visited blocks."""
+    from hbsattn_amd.workloads import Workload, count_work
+    from oracle.dense import hbsa_oracle
+
+    ratio = w.q.shape[1] // w.k.shape[1]
+    cu_nqb, cu_nkb = w.q_meta[3].tolist(), w.k_meta[3].tolist()
+    threads = torch.get_num_threads()
+    done_flops, spent, pairs = 0.0, 0.0, 0
+    tokens = ""
+    for b in range(len(w.cu_q) - 1):
+        qs, qe, ks, ke = w.cu_q[b], w.cu_q[b + 1], w.cu_k[b], w.cu_k[b + 1]
+        tokens = f"{qe - qs} q x {ke - ks} k tokens"
+        for hk in range(w.k.shape[1]):
+            q_heads = list(range(hk * ratio, (hk + 1) * ratio))
+            q_b = w.q[qs:qe][:, q_heads].cpu()
+            k_b, v_b = w.k[ks:ke][:, hk:hk + 1].cpu(), w.v[ks:ke][:, hk:hk + 1].cpu()
+            m_b = w.block_mask[hk:hk + 1, cu_nqb[b]:cu_nqb[b + 1], cu_nkb[b]:cu_nkb[b + 1]].cpu()
+            sub = Workload("sample", q_b, k_b, v_b, [0, qe - qs], [0, ke - ks], None, None, m_b, w.q_block_size,
+                           w.k_block_size, w.causal, w.softmax_scale)
+            t0 = time.perf_counter()
+            hbsa_oracle(q_b, k_b, v_b, sub.cu_q, sub.cu_k, m_b, w.q_block_size, w.k_block_size, w.causal,
+                        w.softmax_scale)
+            spent += time.perf_counter() - t0
+            done_flops += count_work(sub)["flops"]
+            pairs += 1
+            if spent >= budget_s:
+                break
+        if spent >= budget_s:
+            break
+    return {
+        "value": done_flops / spent / 1e12,
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"first {pairs} (sequence, kv head) pairs of the workload in sequence-major order (last one {tokens}, "
+                  f"{ratio} q head(s) per kv head), fp32 masked-dense torch oracle, {spent:.1f} s; effective FLOPs "
+                  "counted over the sample's visited blocks like the GPU figure",
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="C2", choices=sorted(DESCRIPTIONS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-target", action="store_true", help="skip the extra measurement at the 32K target shape")
+    ap.add_argument("--cpu-budget", type=float, default=20.0)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; sequences and kv heads shard with no exchange, "
+                 "so --gpus N>1 is not measured here (use --gpus 1)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+
+    w, res = measure(a.workload, a.steps, a.warmup)
+    line = {
+        "metric": "effective TFLOP/s over kept blocks, block-sparse attention forward (B8 H32 D128)",
+        "value": res["tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": DESCRIPTIONS[a.workload], "timing": "K calls between two synchronisations, "
+                   "block metadata precomputed; pre-pass + attention kernel per call"},
+        "roofline": res["roofline"],
+        "detail": {k: res[k] for k in ("per_call_sync_ms", "attention_kernel_ms", "prepass_ms", "tflops_exact_elements",
+                                       "flops", "bytes", "visited_pairs")},
+    }
+    if not a.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(w, a.cpu_budget)
+    del w
+    torch.cuda.empty_cache()
+    if not a.no_target and a.workload != "T":
+        _, t = measure("T", a.steps, a.warmup)
+        line["target_shape"] = {"workload": DESCRIPTIONS["T"], "ms_per_step": t["ms_per_step"], "tflops": t["tflops"],
+                                "attention_kernel_ms": t["attention_kernel_ms"], "roofline": t["roofline"],
+                                "goal": ">= 0.50 of bf16 dense MFMA peak"}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -40,6 +40,11 @@ def load() -> ctypes.CDLL:
     lib.hbsa_fwd.restype = ctypes.c_int
     lib.hbsa_fwd.argtypes = ([vp] * 11 + [ctypes.c_size_t] + [ctypes.c_int32] * 12 + [ctypes.c_float]
                              + [ctypes.POINTER(ctypes.c_int64), vp])
+    i64p = ctypes.POINTER(ctypes.c_int64)
+    lib.hbsa_fwd_prepare.restype = ctypes.c_int
+    lib.hbsa_fwd_prepare.argtypes = [vp] * 7 + [ctypes.c_size_t] + [ctypes.c_int32] * 7 + [i64p, vp]
+    lib.hbsa_fwd_run.restype = ctypes.c_int
+    lib.hbsa_fwd_run.argtypes = [vp] * 5 + [ctypes.c_size_t] + [ctypes.c_int32] * 11 + [ctypes.c_float, i64p, vp]
     _lib = lib
     return lib
 

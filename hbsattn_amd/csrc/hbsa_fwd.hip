@@ -481,19 +481,50 @@ size_t hbsa_fwd_workspace_bytes(int32_t nhead_k, int32_t num_q_block, int32_t nu
   return info + bits;
 }
 
-int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32_t *cu_q_seqlens,
-             const int32_t *cu_k_seqlens, const uint8_t *block_mask, const int32_t *q_block_to_batch,
-             const int32_t *cu_num_q_block, const int32_t *cu_num_k_block, void *workspace,
-             size_t workspace_bytes, int32_t dtype, int32_t batch, int32_t total_q, int32_t total_k,
-             int32_t nhead_q, int32_t nhead_k, int32_t headdim, int32_t num_q_block, int32_t num_k_block,
-             int32_t q_block_size, int32_t k_block_size, int32_t causal, float softmax_scale,
-             const int64_t *strides, void *stream) {
+int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens, const uint8_t *block_mask,
+                     const int32_t *q_block_to_batch, const int32_t *cu_num_q_block, const int32_t *cu_num_k_block,
+                     void *workspace, size_t workspace_bytes, int32_t batch, int32_t nhead_k, int32_t num_q_block,
+                     int32_t num_k_block, int32_t q_block_size, int32_t k_block_size, int32_t causal,
+                     const int64_t *mask_strides, void *stream) {
   g_err[0] = 0;
-  if (batch < 0 || total_q < 0 || total_k < 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "negative size");
-  if (total_q == 0 || num_q_block == 0 || nhead_q == 0) return 0;  // nothing to write
-  if (!q || !k || !v || !out || !cu_q_seqlens || !cu_k_seqlens || !block_mask || !q_block_to_batch ||
-      !cu_num_q_block || !cu_num_k_block || !workspace || !strides)
+  if (batch < 0 || num_q_block < 0 || num_k_block < 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "negative size");
+  if (num_q_block == 0) return 0;
+  if (!cu_q_seqlens || !cu_k_seqlens || !block_mask || !q_block_to_batch || !cu_num_q_block || !cu_num_k_block ||
+      !workspace || !mask_strides)
     return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer argument");
+  if (nhead_k <= 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "nhead_k must be positive");
+  if (q_block_size <= 0 || k_block_size <= 0 || q_block_size % 16 || k_block_size % 16)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "q_block_size (%d) and k_block_size (%d) must be positive multiples of 16",
+                q_block_size, k_block_size);
+  if (num_k_block <= 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "no keys");
+  if (nhead_k > 65535) return fail(HBSA_ERR_UNSUPPORTED, "nhead_k %d > 65535", nhead_k);
+  if ((uintptr_t)workspace & 255) return fail(HBSA_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
+  const size_t need = hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block);
+  if (workspace_bytes < need)
+    return fail(HBSA_ERR_WORKSPACE_TOO_SMALL, "workspace %zu bytes < required %zu", workspace_bytes, need);
+
+  PrepParams pp;
+  pp.cu_q = cu_q_seqlens; pp.cu_k = cu_k_seqlens; pp.q_block_to_batch = q_block_to_batch;
+  pp.cu_num_q_block = cu_num_q_block; pp.cu_num_k_block = cu_num_k_block;
+  pp.mask = block_mask; pp.ms_h = mask_strides[0]; pp.ms_q = mask_strides[1]; pp.ms_k = mask_strides[2];
+  pp.info = (QBlockInfo *)workspace;
+  pp.bits = (uint32_t *)((char *)workspace + align_up((size_t)num_q_block * sizeof(QBlockInfo), 256));
+  pp.nqb = num_q_block; pp.qbs = q_block_size; pp.kbs = k_block_size; pp.wpr = words_per_row(num_k_block);
+  pp.causal = causal ? 1 : 0;
+  hipLaunchKernelGGL(hbsa_prep_kernel, dim3((num_q_block + 3) / 4, nhead_k), dim3(kThreads), 0, (hipStream_t)stream, pp);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail((int)e, "hbsa_prep_kernel launch: %s", hipGetErrorString(e));
+  return 0;
+}
+
+int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out, const void *workspace, size_t workspace_bytes,
+                 int32_t dtype, int32_t total_q, int32_t total_k, int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+                 int32_t num_q_block, int32_t num_k_block, int32_t q_block_size, int32_t k_block_size, int32_t causal,
+                 float softmax_scale, const int64_t *strides, void *stream) {
+  g_err[0] = 0;
+  if (total_q < 0 || total_k < 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "negative size");
+  if (total_q == 0 || num_q_block == 0 || nhead_q == 0) return 0;  // nothing to write
+  if (!q || !k || !v || !out || !workspace || !strides) return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer argument");
   if (nhead_k <= 0 || nhead_q % nhead_k != 0)
     return fail(HBSA_ERR_INVALID_ARGUMENT, "nhead_q (%d) must be divisible by nhead_k (%d)", nhead_q, nhead_k);
   if (q_block_size <= 0 || k_block_size <= 0 || q_block_size % 16 || k_block_size % 16)
@@ -516,27 +547,14 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32
   if (workspace_bytes < need)
     return fail(HBSA_ERR_WORKSPACE_TOO_SMALL, "workspace %zu bytes < required %zu", workspace_bytes, need);
 
-  hipStream_t st = (hipStream_t)stream;
-  const int wpr = words_per_row(num_k_block);
-  QBlockInfo *info = (QBlockInfo *)workspace;
-  uint32_t *bits = (uint32_t *)((char *)workspace + align_up((size_t)num_q_block * sizeof(QBlockInfo), 256));
-
-  PrepParams pp;
-  pp.cu_q = cu_q_seqlens; pp.cu_k = cu_k_seqlens; pp.q_block_to_batch = q_block_to_batch;
-  pp.cu_num_q_block = cu_num_q_block; pp.cu_num_k_block = cu_num_k_block;
-  pp.mask = block_mask; pp.ms_h = strides[8]; pp.ms_q = strides[9]; pp.ms_k = strides[10];
-  pp.info = info; pp.bits = bits;
-  pp.nqb = num_q_block; pp.qbs = q_block_size; pp.kbs = k_block_size; pp.wpr = wpr; pp.causal = causal ? 1 : 0;
-  hipLaunchKernelGGL(hbsa_prep_kernel, dim3((num_q_block + 3) / 4, nhead_k), dim3(kThreads), 0, st, pp);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return fail((int)e, "hbsa_prep_kernel launch: %s", hipGetErrorString(e));
-
   FwdParams fp;
   fp.q = (const char *)q; fp.k = (const char *)k; fp.v = (const char *)v; fp.out = (char *)out;
-  fp.info = info; fp.bits = bits;
+  fp.info = (const QBlockInfo *)workspace;
+  fp.bits = (const uint32_t *)((const char *)workspace + align_up((size_t)num_q_block * sizeof(QBlockInfo), 256));
   fp.q_s = strides[0] * 2; fp.q_h = strides[1] * 2; fp.k_s = strides[2] * 2; fp.k_h = strides[3] * 2;
   fp.v_s = strides[4] * 2; fp.v_h = strides[5] * 2; fp.o_s = strides[6] * 2; fp.o_h = strides[7] * 2;
-  fp.nqb = num_q_block; fp.ratio = nhead_q / nhead_k; fp.kbs = k_block_size; fp.wpr = wpr; fp.causal = causal ? 1 : 0;
+  fp.nqb = num_q_block; fp.ratio = nhead_q / nhead_k; fp.kbs = k_block_size; fp.wpr = words_per_row(num_k_block);
+  fp.causal = causal ? 1 : 0;
   fp.wps = (q_block_size + kWaveRows - 1) / kWaveRows;
   fp.nsub = (fp.ratio * fp.wps + 3) / 4;
   fp.q_sign = softmax_scale < 0.f ? 0x80008000u : 0u;
@@ -547,12 +565,46 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32
   const long long grid = (long long)nhead_k * num_q_block * fp.nsub;
   if (grid > 0x7fffffffLL) return fail(HBSA_ERR_UNSUPPORTED, "too many work items (%lld)", grid);
 
+  hipStream_t st = (hipStream_t)stream;
   const bool bf = dtype == HBSA_DTYPE_BF16;
   switch (headdim) {
     case 32: return bf ? launch_fwd<32, ElemBF16>(fp, (int)grid, st) : launch_fwd<32, ElemF16>(fp, (int)grid, st);
     case 64: return bf ? launch_fwd<64, ElemBF16>(fp, (int)grid, st) : launch_fwd<64, ElemF16>(fp, (int)grid, st);
     default: return bf ? launch_fwd<128, ElemBF16>(fp, (int)grid, st) : launch_fwd<128, ElemF16>(fp, (int)grid, st);
   }
+}
+
+int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32_t *cu_q_seqlens,
+             const int32_t *cu_k_seqlens, const uint8_t *block_mask, const int32_t *q_block_to_batch,
+             const int32_t *cu_num_q_block, const int32_t *cu_num_k_block, void *workspace,
+             size_t workspace_bytes, int32_t dtype, int32_t batch, int32_t total_q, int32_t total_k,
+             int32_t nhead_q, int32_t nhead_k, int32_t headdim, int32_t num_q_block, int32_t num_k_block,
+             int32_t q_block_size, int32_t k_block_size, int32_t causal, float softmax_scale,
+             const int64_t *strides, void *stream) {
+  g_err[0] = 0;
+  if (total_q == 0 || num_q_block == 0 || nhead_q == 0) return 0;
+  if (!strides) return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer argument");
+  // Validate the main launch before queueing anything, so a refused call leaves no work behind.
+  if (!q || !k || !v || !out) return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer argument");
+  if (nhead_k <= 0 || nhead_q % nhead_k != 0)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "nhead_q (%d) must be divisible by nhead_k (%d)", nhead_q, nhead_k);
+  if (headdim != 32 && headdim != 64 && headdim != 128)
+    return fail(HBSA_ERR_UNSUPPORTED, "headdim %d not in {32, 64, 128}", headdim);
+  if (dtype != HBSA_DTYPE_BF16 && dtype != HBSA_DTYPE_F16)
+    return fail(HBSA_ERR_UNSUPPORTED, "dtype code %d not supported", dtype);
+  if (!std::isfinite(softmax_scale)) return fail(HBSA_ERR_INVALID_ARGUMENT, "softmax_scale is not finite");
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "q/k/v/out must be 16-byte aligned");
+  for (int i = 0; i < 8; ++i)
+    if (strides[i] % 8 != 0)
+      return fail(HBSA_ERR_INVALID_ARGUMENT, "stride %d (%lld elements) is not a multiple of 8 (16-byte rows)", i,
+                  (long long)strides[i]);
+  int rc = hbsa_fwd_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_to_batch, cu_num_q_block, cu_num_k_block,
+                            workspace, workspace_bytes, batch, nhead_k, num_q_block, num_k_block, q_block_size,
+                            k_block_size, causal, strides + 8, stream);
+  if (rc != 0) return rc;
+  return hbsa_fwd_run(q, k, v, out, workspace, workspace_bytes, dtype, total_q, total_k, nhead_q, nhead_k, headdim,
+                      num_q_block, num_k_block, q_block_size, k_block_size, causal, softmax_scale, strides, stream);
 }
 
 }  // extern "C"

@@ -38,13 +38,55 @@ def _pad_headdim(t: torch.Tensor, d_pad: int) -> torch.Tensor:
     return out
 
 
-def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, softmax_scale,
-                 num_q_block, q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block) -> torch.Tensor:
-    """Host launcher: checks, scratch allocation and one call through the C ABI.  No device
-    synchronisation happens here."""
+class PreparedMask:
+    """Result of the pre-pass for one (block_mask, sequence boundaries, block sizes, causal)
+    combination: the device scratch the attention kernel reads.  Reusable across calls that
+    share those, e.g. the layers of a model that share one sparsity pattern."""
+
+    def __init__(self, workspace, nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, causal):
+        self.workspace = workspace
+        self.nhead_k = nhead_k
+        self.num_q_block = num_q_block
+        self.num_k_block = num_k_block
+        self.q_block_size = q_block_size
+        self.k_block_size = k_block_size
+        self.causal = bool(causal)
+
+
+def _check_block_sizes(q_block_size, k_block_size):
+    assert q_block_size > 0 and k_block_size > 0 and q_block_size % 16 == 0 and k_block_size % 16 == 0, \
+        "q_block_size and k_block_size must be integer multiples of 16."
+
+
+def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, num_q_block,
+                 q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block) -> PreparedMask:
+    """Runs the pre-pass kernel (``hbsa_fwd_prepare``) on the current stream."""
+    if not block_mask.is_cuda:
+        raise RuntimeError("hbsattn_amd runs on MI355X only: block_mask must be a CUDA(HIP) tensor; there is no CPU path")
+    _check_block_sizes(q_block_size, k_block_size)
+    lib = _lib.load()
+    dev = block_mask.device
+    nhead_k = block_mask.shape[0]
+    ws_bytes = int(lib.hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block))
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    cu_q, cu_k = _as_int32(cu_q_seqlens), _as_int32(cu_k_seqlens)
+    qb2b, cu_nqb, cu_nkb = _as_int32(q_block_to_batch), _as_int32(cu_num_q_block), _as_int32(cu_num_k_block)
+    mstr = (ctypes.c_int64 * 3)(*block_mask.stride())
+    with torch.cuda.device(dev):
+        rc = lib.hbsa_fwd_prepare(cu_q.data_ptr(), cu_k.data_ptr(), block_mask.data_ptr(), qb2b.data_ptr(),
+                                  cu_nqb.data_ptr(), cu_nkb.data_ptr(), workspace.data_ptr(), ws_bytes, cu_q.numel() - 1,
+                                  nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, int(bool(causal)), mstr,
+                                  torch.cuda.current_stream().cuda_stream)
+    if rc != 0:
+        raise RuntimeError(f"hbsa_fwd_prepare failed (code {rc}): {_lib.last_error()}")
+    return PreparedMask(workspace, nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, causal)
+
+
+def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale) -> torch.Tensor:
+    """Runs the attention kernel (``hbsa_fwd_run``) on the current stream from a prepared mask."""
     if not q.is_cuda:
         raise RuntimeError("hbsattn_amd runs on MI355X only: q/k/v must be CUDA(HIP) tensors; there is no CPU path")
-    if not (k.device == q.device and v.device == q.device and block_mask.device == q.device):
+    if not (k.device == q.device and v.device == q.device and prepared.workspace.device == q.device):
         raise RuntimeError("q, k, v and block_mask must live on the same device")
     if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
         raise ValueError("q, k, v must have shape (total_tokens, nheads, headdim)")
@@ -56,9 +98,9 @@ def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, 
     total_k, nhead_k = k.shape[0], k.shape[1]
     if k.shape[2] != headdim or v.shape != k.shape:
         raise ValueError("k and v must have shape (total_k, nhead_k, headdim) with q's headdim")
+    if nhead_k != prepared.nhead_k:
+        raise ValueError("k has a different number of heads than the prepared block_mask")
     assert nhead_q % nhead_k == 0, "nhead_q must be divisible by nhead_k (for GQA)"
-    assert q_block_size > 0 and k_block_size > 0 and q_block_size % 16 == 0 and k_block_size % 16 == 0, \
-        "q_block_size and k_block_size must be integer multiples of 16."
     if headdim > _NATIVE_HEADDIMS[-1]:
         raise NotImplementedError(f"hbsattn_amd: headdim {headdim} > {_NATIVE_HEADDIMS[-1]} is not supported")
     scale = float(softmax_scale) if softmax_scale is not None else headdim ** -0.5
@@ -67,7 +109,6 @@ def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, 
     out = torch.empty((total_q, nhead_q, headdim), dtype=q.dtype, device=q.device)
     if total_q == 0:
         return out
-
     d_run = next(d for d in _NATIVE_HEADDIMS if d >= headdim)
     if d_run != headdim:  # zero columns add nothing to q.k and give zero output columns
         q, k, v = _pad_headdim(q, d_run), _pad_headdim(k, d_run), _pad_headdim(v, d_run)
@@ -77,32 +118,35 @@ def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, 
         k = k if _rows_ok(k) else k.contiguous()
         v = v if _rows_ok(v) else v.contiguous()
         out_run = out
-
-    cu_q = _as_int32(cu_q_seqlens)
-    cu_k = _as_int32(cu_k_seqlens)
-    qb2b = _as_int32(q_block_to_batch)
-    cu_nqb = _as_int32(cu_num_q_block)
-    cu_nkb = _as_int32(cu_num_k_block)
-    batch = cu_q.numel() - 1
-
-    ws_bytes = int(lib.hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block))
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
-    strides = (ctypes.c_int64 * 11)(q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
-                                    out_run.stride(0), out_run.stride(1), *block_mask.stride())
+    strides = (ctypes.c_int64 * 8)(q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+                                   out_run.stride(0), out_run.stride(1))
+    ws = prepared.workspace
     with torch.cuda.device(q.device):
-        stream = torch.cuda.current_stream().cuda_stream
-        rc = lib.hbsa_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out_run.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),
-                          block_mask.data_ptr(), qb2b.data_ptr(), cu_nqb.data_ptr(), cu_nkb.data_ptr(),
-                          workspace.data_ptr(), ws_bytes, _DTYPE_CODES[q.dtype], batch, total_q, total_k, nhead_q,
-                          nhead_k, d_run, num_q_block, num_k_block, q_block_size, k_block_size, int(bool(causal)),
-                          scale, strides, stream)
+        rc = lib.hbsa_fwd_run(q.data_ptr(), k.data_ptr(), v.data_ptr(), out_run.data_ptr(), ws.data_ptr(), ws.numel(),
+                              _DTYPE_CODES[q.dtype], total_q, total_k, nhead_q, nhead_k, d_run, prepared.num_q_block,
+                              prepared.num_k_block, prepared.q_block_size, prepared.k_block_size, int(prepared.causal),
+                              scale, strides, torch.cuda.current_stream().cuda_stream)
     if rc != 0:
-        raise RuntimeError(f"hbsa_fwd failed (code {rc}): {_lib.last_error()}")
-    # The launches are queued on `stream`; torch's caching allocator keeps `workspace` and any
-    # padded copies alive until work queued on that stream before their release has run.
+        raise RuntimeError(f"hbsa_fwd_run failed (code {rc}): {_lib.last_error()}")
+    # The launch is queued on the current stream; torch's caching allocator keeps padded copies
+    # alive until work queued on that stream before their release has run.
     if out_run is not out:
         out.copy_(out_run[:, :, :headdim])
     return out
+
+
+def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, softmax_scale,
+                 num_q_block, q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block) -> torch.Tensor:
+    """Host launcher: checks, scratch allocation, pre-pass and attention kernel through the C ABI.
+    No device synchronisation happens here."""
+    if not q.is_cuda:
+        raise RuntimeError("hbsattn_amd runs on MI355X only: q/k/v must be CUDA(HIP) tensors; there is no CPU path")
+    if block_mask.device != q.device:
+        raise RuntimeError("q, k, v and block_mask must live on the same device")
+    assert q.shape[1] % k.shape[1] == 0, "nhead_q must be divisible by nhead_k (for GQA)"
+    prepared = hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, num_q_block,
+                            q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block)
+    return hbsa_run(q, k, v, prepared, softmax_scale)
 
 
 class _HBSAttentionFunction(torch.autograd.Function):

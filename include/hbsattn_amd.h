@@ -89,6 +89,40 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out,
              int32_t causal, float softmax_scale,
              const int64_t *strides, void *stream);
 
+/*
+ * The two halves of hbsa_fwd, for callers that apply one block mask to many q/k/v
+ * (layers or steps sharing a sparsity pattern) or that time the kernels separately.
+ *
+ * hbsa_fwd_prepare runs the pre-pass only: it turns block_mask + sequence boundaries into
+ * the compact work description inside `workspace`.  It replaces the per-program mask scan
+ * of the reference kernel (reference hbsattn/fwd_triton_auto_tile_size.py:153-164: every
+ * program loads one mask byte per k block of its sequence and branches on it).
+ *   mask_strides  int64[3] = { mask_head, mask_qblk, mask_kblk } in elements (bytes)
+ *
+ * hbsa_fwd_run runs the attention kernel from a prepared `workspace` (same sizes, block
+ * sizes and `causal` as the prepare call; q/k/v/out and softmax_scale may differ per call).
+ * It replaces the reference `_fwd_kernel` launch (reference
+ * hbsattn/fwd_triton_auto_tile_size.py:283-308).
+ *   strides       int64[8] = { q_tok, q_head, k_tok, k_head, v_tok, v_head, out_tok, out_head }
+ */
+int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens,
+                     const uint8_t *block_mask,
+                     const int32_t *q_block_to_batch, const int32_t *cu_num_q_block,
+                     const int32_t *cu_num_k_block,
+                     void *workspace, size_t workspace_bytes,
+                     int32_t batch, int32_t nhead_k, int32_t num_q_block, int32_t num_k_block,
+                     int32_t q_block_size, int32_t k_block_size, int32_t causal,
+                     const int64_t *mask_strides, void *stream);
+
+int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out,
+                 const void *workspace, size_t workspace_bytes,
+                 int32_t dtype, int32_t total_q, int32_t total_k,
+                 int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+                 int32_t num_q_block, int32_t num_k_block,
+                 int32_t q_block_size, int32_t k_block_size,
+                 int32_t causal, float softmax_scale,
+                 const int64_t *strides, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

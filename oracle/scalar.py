@@ -36,7 +36,7 @@ def load() -> ctypes.CDLL:
         lib.hbsa_oracle_calculate_blocks.argtypes = [i32p, ctypes.c_int32, ctypes.c_int32, i32p, i32p, i32p]
         lib.hbsa_oracle_fwd.restype = ctypes.c_int
         lib.hbsa_oracle_fwd.argtypes = [f32p, f32p, f32p, f32p, i32p, i32p, u8p] + [ctypes.c_int32] * 9 + [
-            ctypes.c_int32, ctypes.c_double, ctypes.c_int64, ctypes.c_int64]
+            ctypes.c_double, ctypes.c_int64, ctypes.c_int64]
         lib.hbsa_oracle_max_threads.restype = ctypes.c_int
         _lib = lib
     return _lib

@@ -1,0 +1,82 @@
+"""The C-ABI library loads without a GPU and exports every function the header declares.
+Only host-side entry points and argument validation are exercised here (no kernel runs)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from hbsattn_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hbsattn_amd.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hbsa_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared_functions()
+    assert {"hbsa_abi_version", "hbsa_last_error", "hbsa_fwd_workspace_bytes", "hbsa_fwd"} <= set(names)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in _declared_functions():
+        assert hasattr(lib, name), f"{name} declared in include/hbsattn_amd.h but not exported"
+
+
+def test_abi_version_matches_header():
+    lib = _lib.load()
+    version = int(re.search(r"#define HBSA_ABI_VERSION (\d+)", open(HEADER).read()).group(1))
+    assert lib.hbsa_abi_version() == version == _lib.ABI_VERSION
+
+
+def test_workspace_bytes_is_host_only_and_monotone():
+    lib = _lib.load()
+    a = lib.hbsa_fwd_workspace_bytes(2, 5, 12)
+    b = lib.hbsa_fwd_workspace_bytes(32, 2048, 2048)
+    c = lib.hbsa_fwd_workspace_bytes(32, 4096, 4096)
+    assert 0 < a < b < c
+    assert a % 256 == 0 and b % 256 == 0
+    # one bit per k block per (kv head, q block) plus a 32-byte record per q block
+    assert b >= 32 * 2048 * (2048 // 8) + 2048 * 32
+    assert c < 80 * 2 ** 20
+
+
+def _call_fwd(lib, **over):
+    strides = (ctypes.c_int64 * 11)(4096, 128, 4096, 128, 4096, 128, 4096, 128, 1, 1, 1)
+    a = dict(q=256, k=256, v=256, out=256, cu_q=256, cu_k=256, mask=256, qb2b=256, cu_nqb=256, cu_nkb=256, ws=256,
+             ws_bytes=1 << 30, dtype=0, batch=1, total_q=128, total_k=128, hq=32, hk=32, d=128, nqb=1, nkb=1, qbs=128,
+             kbs=128, causal=1, scale=0.1)
+    a.update(over)
+    return lib.hbsa_fwd(a["q"], a["k"], a["v"], a["out"], a["cu_q"], a["cu_k"], a["mask"], a["qb2b"], a["cu_nqb"],
+                        a["cu_nkb"], a["ws"], a["ws_bytes"], a["dtype"], a["batch"], a["total_q"], a["total_k"], a["hq"],
+                        a["hk"], a["d"], a["nqb"], a["nkb"], a["qbs"], a["kbs"], a["causal"], a["scale"], strides, None)
+
+
+@pytest.mark.parametrize("over,code,needle", [
+    (dict(q=None), -1, "null"),
+    (dict(hq=30, hk=4), -1, "divisible"),
+    (dict(qbs=100), -1, "multiples of 16"),
+    (dict(kbs=0), -1, "multiples of 16"),
+    (dict(d=96), -2, "headdim"),
+    (dict(dtype=7), -2, "dtype"),
+    (dict(ws_bytes=16), -3, "workspace"),
+    (dict(q=264), -1, "aligned"),
+    (dict(scale=float("inf")), -1, "finite"),
+])
+def test_argument_validation_reports_errors_without_touching_the_gpu(over, code, needle):
+    lib = _lib.load()
+    rc = _call_fwd(lib, **over)
+    assert rc == code
+    assert needle in _lib.last_error()
+
+
+def test_empty_problem_is_a_no_op():
+    lib = _lib.load()
+    assert _call_fwd(lib, total_q=0, q=None) == 0
+    assert _lib.last_error() == ""
