@@ -66,6 +66,8 @@ struct QBlockInfo {
   int32_t kmax;        // exclusive in-sequence bound of keys any row of the block may see
 };
 
+struct Sched;
+
 struct PrepParams {
   const int32_t *cu_q, *cu_k, *q_block_to_batch, *cu_num_q_block, *cu_num_k_block;
   const uint8_t *mask;
@@ -87,6 +89,8 @@ struct FwdParams {
   uint32_t q_sign;  // 0x80008000 when softmax_scale < 0 (Q is negated, |scale| used)
   float c;        // |softmax_scale| * log2(e)
   float lag;      // kLazyRescaleLog2 / c, in raw score units
+  int32_t nhead_k;
+  struct Sched *sched;
 };
 
 // --------------------------------------------------------------------------------------
@@ -147,60 +151,6 @@ struct ElemF16 {
   }
 };
 
-// Walks the kept k blocks of one (kv head, q block): adjacent kept blocks form a run of
-// keys; runs are handed out in tiles of kTileKeys.  All state is wavefront-uniform.  The
-// row's bit words live in a VGPR (lane i holds word i of the current 64-word window) and
-// are fetched with v_readlane, so stepping costs no memory latency.
-struct TileWalker {
-  const uint32_t *bits;
-  int nwords, kbs, kmax, lane;
-  int window;     // index of the 64-word window held in `held`
-  uint32_t held;  // lane i: word window*64 + i (0 past the end of the row)
-  int blk;        // next k block (in-sequence) to examine
-  int pos, end;   // remaining keys of the current run, in-sequence positions
-
-  __device__ __forceinline__ void init(const uint32_t *row, int nwords_, int kbs_, int kmax_, int lane_) {
-    bits = row; nwords = nwords_; kbs = kbs_; kmax = kmax_; lane = lane_;
-    window = 0;
-    held = lane < nwords ? row[lane] : 0u;
-    blk = 0; pos = 0; end = 0;
-  }
-  __device__ __forceinline__ uint32_t word(int w) {
-    if ((w >> 6) != window) {
-      window = w >> 6;
-      const int i = window * 64 + lane;
-      held = i < nwords ? bits[i] : 0u;
-    }
-    return (uint32_t)__builtin_amdgcn_readlane((int)held, w & 63);
-  }
-  __device__ __forceinline__ bool next(int &kpos, int &valid) {
-    if (pos >= end) {
-      int w = blk >> 5;
-      if (w >= nwords) return false;
-      uint32_t cur = word(w) & (~0u << (blk & 31));
-      while (cur == 0) {
-        if (++w >= nwords) return false;
-        cur = word(w);
-      }
-      const int first = w * 32 + __builtin_ctz(cur);
-      uint32_t inv = ~word(w) & (~0u << (first & 31));
-      while (inv == 0) {
-        if (++w >= nwords) break;
-        inv = ~word(w);
-      }
-      const int stop = (w >= nwords) ? nwords * 32 : w * 32 + __builtin_ctz(inv);
-      blk = stop;
-      pos = first * kbs;
-      end = min(stop * kbs, kmax);
-      if (pos >= end) return false;
-    }
-    kpos = pos;
-    valid = min(kTileKeys, end - pos);
-    pos += kTileKeys;
-    return true;
-  }
-};
-
 // exchange-and-combine between lane i and lane i^32
 __device__ __forceinline__ float half_max(float x) {
   const uint32_t u = __builtin_bit_cast(uint32_t, x);
@@ -214,11 +164,139 @@ __device__ __forceinline__ float half_sum(float x) {
 }
 
 // --------------------------------------------------------------------------------------
-// Main kernel.  D = head dim (32, 64 or 128); rows of K/V tiles are D*2 bytes in LDS.
+// Main kernel (persistent).  D = head dim (32, 64 or 128); rows of K/V tiles are D*2 bytes.
+//
+// Scheduling.  The grid is as many workgroups as fit the device at once and every workgroup
+// loops over work items it claims from eight queues, one per XCD (the chip's eight dies, each
+// with its own L2).  Queue v holds, head-major, the items of the kv heads h with h % 8 == v:
+// for each such head every q block of the packed batch from the last to the first (under a
+// causal mask the heaviest blocks of each sequence come first), and for each q block its
+// groups of four wave slots.  The queues need no storage: entry idx of queue v decodes
+// arithmetically, and one atomic counter per queue hands entries out.  A workgroup reads the
+// id of the XCD it runs on from the hardware and drains that XCD's queue, so at any time the
+// workgroups that share an L2 walk the K/V of one (or few) kv heads; when its queue is empty it
+// takes from the other queues, which balances the tail.  A workgroup ends after at most eight
+// consecutive failed claims, one per queue.
+//
+// Division of labour.  Wavefront 0 is also the workgroup's scheduler: one item ahead it
+// claims a queue entry, fetches that item's geometry record and mask bits, and expands the
+// bits into a list of 64-key tiles in LDS (adjacent kept k blocks merge into key runs).  The
+// main loop of every wavefront then only steps through that list: no mask logic, no global
+// metadata loads and no divergent control flow remain on the per-tile path.
+//
+// Pipelining.  K/V tiles stream through two LDS buffers without a bubble at item borders:
+// while the last tile of an item is being computed the first tile of the next item is
+// already on its way and the next item's Q rows are being fetched.
+//
 // LDS: K[2][64][D] then V[2][64][D] (double-buffered 64-key tiles), 16-byte chunks of
 // every row XOR-swizzled so that both the K reads (16 rows x one chunk per 16 lanes) and
-// the transposing V reads (4 rows x 64 bytes per 32 lanes) spread over all banks.
+// the transposing V reads (4 rows x 64 bytes per 32 lanes) spread over all banks; then two
+// item headers and two tile lists.
 // --------------------------------------------------------------------------------------
+struct Sched {
+  uint32_t qnext[8];   // next unclaimed entry of each queue
+  uint32_t pad[56];
+};
+
+__global__ void hbsa_reset_kernel(Sched *s) {
+  if (threadIdx.x < 8) s->qnext[threadIdx.x] = 0;
+}
+
+constexpr int kListCap = 1024;   // tile entries per list; longer items are expanded in chunks
+
+// Item header in LDS (16 ints).
+enum { H_HK = 0, H_QB, H_SUB, H_TOTAL, H_ROW_BEGIN, H_ROWS, H_KEY_BEGIN, H_Q_POS, H_SHIFT, H_WORDS = 16 };
+
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+// A tile entry packs the in-sequence position of the tile's first key (a multiple of 16) and
+// the number of valid keys (1..64).
+__device__ __forceinline__ int pack_tile(int pos, int valid) { return ((pos >> 4) << 6) | (valid - 1); }
+
+// Expands one item's kept-block bits into tile entries [chunk_base, chunk_base + kListCap) of
+// the item's tile sequence, written to list[0..); returns the item's total tile count.
+// Executed by one whole wavefront; `first_words`: lane i holds bit word i of the row.
+__device__ __forceinline__ int build_tile_list(int *list, int chunk_base, const uint32_t *row, int nwords, int kbs,
+                                                int kmax, uint32_t first_words, int lane) {
+  if (kmax <= 0 || nwords <= 0) return 0;
+  int total = 0;
+  if ((kbs & 63) == 0) {
+    // Blocks are whole tiles: every kept block yields kbs/64 tiles, the one holding key
+    // kmax-1 possibly fewer.  Lane i expands word i; offsets come from a wavefront scan.
+    const int tpb = kbs >> 6;
+    const int j_last = (kmax - 1) / kbs;
+    const int t_last = (kmax - j_last * kbs + 63) >> 6;
+    for (int win = 0; win * 64 < nwords; ++win) {
+      const int widx = win * 64 + lane;
+      uint32_t w = win == 0 ? (lane < nwords ? first_words : 0u) : (widx < nwords ? row[widx] : 0u);
+      int cnt = __builtin_popcount(w) * tpb;
+      if ((j_last >> 5) == widx && ((w >> (j_last & 31)) & 1u)) cnt -= tpb - t_last;
+      int incl = cnt;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+      }
+      int off = total + incl - cnt - chunk_base;
+      while (w) {
+        const int j = widx * 32 + __builtin_ctz(w);
+        w &= w - 1;
+        for (int t = 0; t < tpb; ++t) {
+          const int pos = j * kbs + 64 * t;
+          if (pos < kmax) {
+            if (off >= 0 && off < kListCap) list[off] = pack_tile(pos, min(kTileKeys, kmax - pos));
+            ++off;
+          }
+        }
+      }
+      total += __builtin_amdgcn_readlane(incl, 63);
+    }
+  } else {
+    // General block sizes: walk the runs of adjacent kept blocks serially (wavefront-uniform).
+    int window = 0;
+    uint32_t held = lane < nwords ? first_words : 0u;
+    auto word = [&](int w) -> uint32_t {
+      if ((w >> 6) != window) {
+        window = w >> 6;
+        const int i = window * 64 + lane;
+        held = i < nwords ? row[i] : 0u;
+      }
+      return (uint32_t)__builtin_amdgcn_readlane((int)held, w & 63);
+    };
+    int blk = 0;
+    for (;;) {
+      int w = blk >> 5;
+      if (w >= nwords) break;
+      uint32_t cur = word(w) & (~0u << (blk & 31));
+      while (cur == 0) {
+        if (++w >= nwords) break;
+        cur = word(w);
+      }
+      if (w >= nwords) break;
+      const int first = w * 32 + __builtin_ctz(cur);
+      uint32_t inv = ~word(w) & (~0u << (first & 31));
+      while (inv == 0) {
+        if (++w >= nwords) break;
+        inv = ~word(w);
+      }
+      const int stop = (w >= nwords) ? nwords * 32 : w * 32 + __builtin_ctz(inv);
+      blk = stop;
+      const int end = min(stop * kbs, kmax);
+      for (int pos = first * kbs; pos < end; pos += kTileKeys) {
+        const int off = total - chunk_base;
+        if (lane == 0 && off >= 0 && off < kListCap) list[off] = pack_tile(pos, min(kTileKeys, end - pos));
+        ++total;
+      }
+      if (end >= kmax) break;
+    }
+  }
+  return total;
+}
+
 template <int D, typename E>
 __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   constexpr int RB = D * 2;            // row bytes
@@ -232,91 +310,124 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   char *lds_k = lds;
   char *lds_v = lds + 2 * TILE_BYTES;
+  int *lds_hdr = (int *)(lds + 4 * TILE_BYTES);     // [2][H_WORDS]
+  int *lds_list = lds_hdr + 2 * H_WORDS;            // [2][kListCap]
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g32 = lane >> 5;   // which half of the wavefront
   const int l32 = lane & 31;   // query within the wave slot / key row within a sub-tile
 
-  // ---- work item: head-major, q blocks from the end of the packed batch backwards so
-  // that under a causal mask the heaviest blocks of every sequence are issued first.
-  const int bid = blockIdx.x;
-  const int sub = bid % p.nsub;
-  const int t = bid / p.nsub;
-  const int qb = p.nqb - 1 - (t % p.nqb);
-  const int hk = t / p.nqb;
+  // ------------------------------------------------------------------ scheduler (wavefront 0)
+  const int nq = p.nhead_k < 8 ? p.nhead_k : 8;                       // queues that hold work
+  const int home = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7;    // HW_REG_XCC_ID
+  const int first_queue = home < nq ? home : home % nq;
+  int tries = 0;                    // queues found empty so far
+  uint32_t pending = 0xffffffffu;   // queue index claimed for the item after the staged one
+  int st_hk = -1, st_qb = 0, st_sub = 0;   // staged item: claimed, records fetched, list not built
+  uint32_t st_info = 0, st_bits = 0;       // lane i: word i of its QBlockInfo / of its bit row
 
-  const QBlockInfo info = p.info[qb];
-  const int slot = sub * 4 + wave;
-  const int head_in_group = slot / p.wps;
-  const int row0 = (slot % p.wps) * kWaveRows;          // first row of this wave inside the q block
-  const int nrows = min(kWaveRows, info.rows - row0);
-  const bool active = head_in_group < p.ratio && nrows > 0;
-  const int hq = hk * p.ratio + head_in_group;
+  auto queue_len = [&](int v) -> uint32_t {
+    const int heads = v < p.nhead_k ? (p.nhead_k - v + 7) / 8 : 0;
+    return (uint32_t)heads * (uint32_t)p.nqb * (uint32_t)p.nsub;
+  };
+  auto claim = [&]() -> uint32_t {   // the value is looked at an item later, so its latency is hidden
+    uint32_t r = 0xffffffffu;
+    if (tries < 8) {
+      if (lane == 0) r = atomicAdd(&p.sched->qnext[(first_queue + tries) & 7], 1u);
+    }
+    return r;
+  };
+  // turn `pending` into the staged item (claiming again from the next queues when the one it
+  // came from is exhausted) and start fetching the item's records
+  auto stage = [&]() {
+    uint32_t claimed = (uint32_t)__builtin_amdgcn_readfirstlane((int)pending);
+    st_hk = -1;
+    while (tries < 8) {
+      const int v = (first_queue + tries) & 7;
+      if (claimed < queue_len(v)) {
+        const uint32_t t = claimed / (uint32_t)p.nsub;
+        st_sub = (int)(claimed % (uint32_t)p.nsub);
+        st_hk = v + 8 * (int)(t / (uint32_t)p.nqb);
+        st_qb = p.nqb - 1 - (int)(t % (uint32_t)p.nqb);
+        break;
+      }
+      if (++tries >= 8) break;
+      uint32_t r = 0;
+      if (lane == 0) r = atomicAdd(&p.sched->qnext[(first_queue + tries) & 7], 1u);
+      claimed = (uint32_t)__builtin_amdgcn_readfirstlane((int)r);
+    }
+    if (st_hk >= 0) {
+      st_info = lane < 8 ? ((const uint32_t *)(p.info + st_qb))[lane] : 0u;
+      st_bits = lane < p.wpr ? p.bits[((size_t)st_hk * p.nqb + st_qb) * p.wpr + lane] : 0u;
+    }
+  };
+  // expand the staged item into list `c` and write its header
+  auto build = [&](int c) {
+    int *hdr = lds_hdr + c * H_WORDS;
+    int total = 0;
+    if (st_hk >= 0) {
+      const int nkblk = __builtin_amdgcn_readlane((int)st_info, 6);
+      const int kmax = __builtin_amdgcn_readlane((int)st_info, 7);
+      total = build_tile_list(lds_list + c * kListCap, 0, p.bits + ((size_t)st_hk * p.nqb + st_qb) * p.wpr,
+                              2 * ((nkblk + 63) >> 6), p.kbs, kmax, st_bits, lane);
+    }
+    if (lane == 0) {
+      hdr[H_HK] = st_hk; hdr[H_QB] = st_qb; hdr[H_SUB] = st_sub; hdr[H_TOTAL] = total;
+    }
+    if (lane < 8) {   // QBlockInfo words: row_begin, rows, key_begin, klen, q_pos, shift, nkblk, kmax
+      const int dst = lane == 0 ? H_ROW_BEGIN : lane == 1 ? H_ROWS : lane == 2 ? H_KEY_BEGIN : lane == 4 ? H_Q_POS
+                      : lane == 5 ? H_SHIFT : -1;
+      if (dst >= 0) hdr[dst] = (int)st_info;
+    }
+  };
 
-  // ---- per-thread source/destination pattern of the tile loads (same for every tile)
+  if (wave == 0) {
+    pending = claim();
+    stage();
+    build(0);
+    pending = claim();
+    stage();
+    pending = claim();
+  }
+  __syncthreads();
+
+  // ------------------------------------------------------------------ per-thread constants
+  // tile loads: thread -> (row, 16-byte chunk) of the tile, same for every tile
   int ld_row[LOADS];
-  int ld_koff[LOADS], ld_voff[LOADS];
+  uint32_t ld_koff[LOADS], ld_voff[LOADS];   // byte offset of the thread's chunk from the tile's first row
+  int ld_kchunk[LOADS], ld_vchunk[LOADS];
 #pragma unroll
   for (int i = 0; i < LOADS; ++i) {
     const int c = (i * 4 + wave) * 64 + lane;
     const int r = c / CPR, pc = c % CPR;
     ld_row[i] = r;
-    ld_koff[i] = (pc ^ ((r / RPG) % CPR)) * 16;
-    ld_voff[i] = (pc ^ ((CPR >= 8) ? (((r / RPG) % (CPR / 4)) << 2) : 0)) * 16;
+    ld_kchunk[i] = (pc ^ ((r / RPG) % CPR)) * 16;
+    ld_vchunk[i] = (pc ^ ((CPR >= 8) ? (((r / RPG) % (CPR / 4)) << 2) : 0)) * 16;
+    ld_koff[i] = (uint32_t)r * (uint32_t)p.k_s + (uint32_t)ld_kchunk[i];
+    ld_voff[i] = (uint32_t)r * (uint32_t)p.v_s + (uint32_t)ld_vchunk[i];
   }
-  const char *kg = p.k + (int64_t)hk * p.k_h;
-  const char *vg = p.v + (int64_t)hk * p.v_h;
-
-  auto issue_loads = [&](int buf, int kpos, int valid) {
-    const int tok0 = info.key_begin + kpos;
-    const int tok_last = tok0 + valid - 1;
+  // kbase / vbase: wavefront-uniform address of the tile's first key row (for this kv head)
+  auto issue_loads = [&](int buf, const char *kbase, const char *vbase, int valid) {
+    if (valid == kTileKeys) {
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-      const int tok = min(tok0 + ld_row[i], tok_last);
-      const int lds_off = buf * TILE_BYTES + (i * 4 + wave) * 1024;
-      __builtin_amdgcn_global_load_lds(HBSA_AS1(kg + (int64_t)tok * p.k_s + ld_koff[i]), HBSA_AS3(lds_k + lds_off), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(HBSA_AS1(vg + (int64_t)tok * p.v_s + ld_voff[i]), HBSA_AS3(lds_v + lds_off), 16, 0, 0);
+      for (int i = 0; i < LOADS; ++i) {
+        const int lds_off = buf * TILE_BYTES + (i * 4 + wave) * 1024;
+        __builtin_amdgcn_global_load_lds(HBSA_AS1(kbase + ld_koff[i]), HBSA_AS3(lds_k + lds_off), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(HBSA_AS1(vbase + ld_voff[i]), HBSA_AS3(lds_v + lds_off), 16, 0, 0);
+      }
+    } else {   // ragged tail of a run: rows past the end re-read the last valid row (masked later)
+#pragma unroll
+      for (int i = 0; i < LOADS; ++i) {
+        const uint32_t r = (uint32_t)min(ld_row[i], valid - 1);
+        const int lds_off = buf * TILE_BYTES + (i * 4 + wave) * 1024;
+        __builtin_amdgcn_global_load_lds(HBSA_AS1(kbase + (r * (uint32_t)p.k_s + (uint32_t)ld_kchunk[i])), HBSA_AS3(lds_k + lds_off), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(HBSA_AS1(vbase + (r * (uint32_t)p.v_s + (uint32_t)ld_vchunk[i])), HBSA_AS3(lds_v + lds_off), 16, 0, 0);
+      }
     }
   };
 
-  TileWalker walk;
-  walk.init(p.bits + ((size_t)hk * p.nqb + qb) * p.wpr, 2 * ((info.nkblk + 63) >> 6), p.kbs, info.kmax, lane);
-
-  int kpos = 0, valid = 0;
-  bool have = walk.next(kpos, valid);
-  if (have) issue_loads(0, kpos, valid);
-
-  // ---- Q^T fragments (B operand): lane holds query l32, d = 16*ks + 8*g32 .. +7
-  short8v qf[KSTEPS];
-  if (active) {
-    const int r = min(row0 + l32, info.rows - 1);
-    const char *qrow = p.q + (int64_t)(info.row_begin + r) * p.q_s + (int64_t)hq * p.q_h + g32 * 16;
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      u32x4 raw = *(const u32x4 *)(qrow + ks * 32);
-      raw ^= p.q_sign;
-      qf[ks] = __builtin_bit_cast(short8v, raw);
-    }
-  } else {
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = (short8v)0;
-  }
-
-  f32x16 o[DT];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
-  float m_run = -INFINITY;  // running reference max, raw (unscaled) score units
-  float l_run = 0.f;        // this lane's share of the row sum
-
-  // causal visibility of this lane's / this wave's rows: key position <= qpos + shift
-  const int lane_kvis = info.q_pos + min(row0 + l32, info.rows - 1) + info.shift;
-  const int wave_kvis_min = info.q_pos + row0 + info.shift;
-  const int wave_kvis_max = info.q_pos + row0 + nrows - 1 + info.shift;
-
-  // ---- per-lane LDS read addresses
+  // per-lane LDS read addresses
   // K (A operand of S^T): row l32 (+32), chunk (2*ks + g32) ^ swz(row)
   const int k_rd = l32 * RB + ((g32 ^ ((l32 / RPG) % CPR)) << 4);
   // V^T (A operand of O^T) through ds_read_b64_tr_b16: within a group of 16 lanes, lane r
@@ -326,114 +437,274 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   const int v_swz = (CPR >= 8) ? (((v_key / RPG) % (CPR / 4)) << 2) : 0;
   const int v_rd = v_key * RB + ((v_lc | v_swz) << 4) + 8 * (lane & 1);
 
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): first tile has landed in LDS
-  __syncthreads();
+  auto hdr_word = [&](int c, int i) { return __builtin_amdgcn_readfirstlane(lds_hdr[c * H_WORDS + i]); };
+  // this wave's slice of an item: q head, first row inside the q block, rows
+  auto q_row_ptr = [&](int hk, int sub, int row_begin, int rows, bool &act, int &hq, int &row0, int &nrows) {
+    const int slot = sub * 4 + wave;
+    const int head_in_group = slot / p.wps;
+    row0 = (slot % p.wps) * kWaveRows;
+    nrows = min(kWaveRows, rows - row0);
+    act = head_in_group < p.ratio && nrows > 0;
+    hq = hk * p.ratio + head_in_group;
+    const int r = min(row0 + l32, rows - 1);
+    return p.q + (int64_t)(row_begin + r) * p.q_s + (int64_t)hq * p.q_h + g32 * 16;
+  };
 
+  // ------------------------------------------------------------------ first item
+  int c = 0;   // list / header of the current item
+  if (hdr_word(0, H_HK) < 0) return;
   int buf = 0;
-  while (have) {
-    int nkpos = 0, nvalid = 0;
-    const bool have_next = walk.next(nkpos, nvalid);
-    if (have_next) issue_loads(buf ^ 1, nkpos, nvalid);
+  {
+    const int total0 = hdr_word(0, H_TOTAL);
+    if (total0 > 0) {
+      const int e = __builtin_amdgcn_readfirstlane(lds_list[0]);
+      const int64_t tok = hdr_word(0, H_KEY_BEGIN) + ((e >> 6) << 4);
+      const int hk = hdr_word(0, H_HK);
+      issue_loads(0, p.k + (int64_t)hk * p.k_h + tok * p.k_s, p.v + (int64_t)hk * p.v_h + tok * p.v_s, (e & 63) + 1);
+    }
+  }
+  short8v qf[KSTEPS];   // Q^T fragments (B operand): lane holds query l32, d = 16*ks + 8*g32 .. +7
+  {
+    bool act; int hq, row0, nrows;
+    const char *qrow = q_row_ptr(hdr_word(0, H_HK), hdr_word(0, H_SUB), hdr_word(0, H_ROW_BEGIN), hdr_word(0, H_ROWS), act,
+                                 hq, row0, nrows);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      u32x4 raw = {0u, 0u, 0u, 0u};
+      if (act) raw = *(const u32x4 *)(qrow + ks * 32);
+      raw ^= p.q_sign;
+      qf[ks] = __builtin_bit_cast(short8v, raw);
+    }
+  }
 
-    if (active && (!p.causal || kpos <= wave_kvis_max)) {
-      const uint32_t kt_base = (uint32_t)(uintptr_t)HBSA_AS3(lds_k + buf * TILE_BYTES);
-      const uint32_t vt_base = (uint32_t)(uintptr_t)HBSA_AS3(lds_v + buf * TILE_BYTES);
-      // ---- S^T = K . Q^T  (two 32-key sub-tiles)
-      f32x16 s[2];
+  for (;;) {   // ------------------------------------------------------ one iteration per work item
+    const int cur_hk = hdr_word(c, H_HK);
+    const int cur_sub = hdr_word(c, H_SUB);
+    const int total = hdr_word(c, H_TOTAL);
+    const int row_begin = hdr_word(c, H_ROW_BEGIN);
+    const int rows = hdr_word(c, H_ROWS);
+    const int key_begin = hdr_word(c, H_KEY_BEGIN);
+    const int q_pos = hdr_word(c, H_Q_POS);
+    const int shift = hdr_word(c, H_SHIFT);
+
+    if (wave == 0) {   // stay one item ahead: expand the staged item, stage the one after it
+      build(c ^ 1);
+      stage();
+      pending = claim();
+    }
+
+    bool active; int hq, row0, nrows;
+    (void)q_row_ptr(cur_hk, cur_sub, row_begin, rows, active, hq, row0, nrows);
+
+    f32x16 o[DT];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) { s[0][i] = 0.f; s[1][i] = 0.f; }
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const uint32_t a = kt_base + (uint32_t)(k_rd ^ (ks * 32));
-        const short8v a0 = *(const __attribute__((address_space(3))) short8v *)(uintptr_t)a;
-        const short8v a1 = *(const __attribute__((address_space(3))) short8v *)(uintptr_t)(a + 32 * RB);
-        s[0] = E::mfma(a0, qf[ks], s[0]);
-        s[1] = E::mfma(a1, qf[ks], s[1]);
+      for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
+    float m_run = -INFINITY;  // running reference max, raw (unscaled) score units
+    float l_run = 0.f;        // this lane's share of the row sum
+
+    // causal visibility of this lane's / this wave's rows: key position <= qpos + shift
+    const int lane_kvis = q_pos + min(row0 + l32, rows - 1) + shift;
+    const int wave_kvis_min = q_pos + row0 + shift;
+    const int wave_kvis_max = q_pos + row0 + nrows - 1 + shift;
+    const char *kg = p.k + (int64_t)cur_hk * p.k_h + (int64_t)key_begin * p.k_s;
+    const char *vg = p.v + (int64_t)cur_hk * p.v_h + (int64_t)key_begin * p.v_s;
+
+    int nxt_hk = -1;          // known once the last tile is reached
+    int chunk_base = 0;
+    for (;;) {   // ---------------------------------------------------- chunks of the tile list (usually one)
+      const int n = min(kListCap, total - chunk_base);
+      int held = 0;           // lane i: entry (window * 64 + i) of the current chunk
+      for (int t = 0; t < n; ++t) {   // ---------------------------------- one iteration per 64-key tile
+        if ((t & 63) == 0) held = (t + lane < n) ? lds_list[c * kListCap + t + lane] : 0;
+        const int e = __builtin_amdgcn_readlane(held, t & 63);
+        const int kpos = (e >> 6) << 4, valid = (e & 63) + 1;
+
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the current tile has landed in LDS
+        __syncthreads();                     // ... for every wave, and the other buffers are free
+
+        const bool last = chunk_base + t + 1 == total;
+        if (t + 1 < n) {
+          int e1;
+          if (((t + 1) & 63) == 0) {
+            const int h1 = (t + 1 + lane < n) ? lds_list[c * kListCap + t + 1 + lane] : 0;
+            e1 = __builtin_amdgcn_readlane(h1, 0);
+          } else {
+            e1 = __builtin_amdgcn_readlane(held, (t + 1) & 63);
+          }
+          const int64_t tok = (e1 >> 6) << 4;
+          issue_loads(buf ^ 1, kg + tok * p.k_s, vg + tok * p.v_s, (e1 & 63) + 1);
+        } else if (last) {
+          nxt_hk = hdr_word(c ^ 1, H_HK);
+          if (nxt_hk >= 0 && hdr_word(c ^ 1, H_TOTAL) > 0) {
+            const int e1 = __builtin_amdgcn_readfirstlane(lds_list[(c ^ 1) * kListCap]);
+            const int64_t tok = hdr_word(c ^ 1, H_KEY_BEGIN) + ((e1 >> 6) << 4);
+            issue_loads(buf ^ 1, p.k + (int64_t)nxt_hk * p.k_h + tok * p.k_s, p.v + (int64_t)nxt_hk * p.v_h + tok * p.v_s,
+                        (e1 & 63) + 1);
+          }
+        }
+
+        const bool compute = active && (!p.causal || kpos <= wave_kvis_max);
+        f32x16 s[2];
+        if (compute) {
+          const uint32_t kt_base = (uint32_t)(uintptr_t)HBSA_AS3(lds_k + buf * TILE_BYTES);
+          // ---- S^T = K . Q^T  (two 32-key sub-tiles)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) { s[0][i] = 0.f; s[1][i] = 0.f; }
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            const uint32_t a = kt_base + (uint32_t)(k_rd ^ (ks * 32));
+            const short8v a0 = *(const __attribute__((address_space(3))) short8v *)(uintptr_t)a;
+            const short8v a1 = *(const __attribute__((address_space(3))) short8v *)(uintptr_t)(a + 32 * RB);
+            s[0] = E::mfma(a0, qf[ks], s[0]);
+            s[1] = E::mfma(a1, qf[ks], s[1]);
+          }
+        }
+        if (last && nxt_hk >= 0) {
+          // Q of this item is no longer needed: fetch the next item's rows under this tile's softmax
+          bool act; int hq1, r01, nr1;
+          const char *qrow = q_row_ptr(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS),
+                                       act, hq1, r01, nr1);
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            u32x4 raw = {0u, 0u, 0u, 0u};
+            if (act) raw = *(const u32x4 *)(qrow + ks * 32);
+            raw ^= p.q_sign;
+            qf[ks] = __builtin_bit_cast(short8v, raw);
+          }
+        }
+        if (compute) {
+          const uint32_t vt_base = (uint32_t)(uintptr_t)HBSA_AS3(lds_v + buf * TILE_BYTES);
+          // ---- edge tiles: ragged run tail and the causal diagonal
+          const bool edge = valid < kTileKeys || (p.causal && kpos + valid - 1 > wave_kvis_min);
+          if (edge) {
+            int lim = valid;
+            if (p.causal) lim = min(lim, lane_kvis - kpos + 1);
+            lim -= 4 * g32;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+              for (int i = 0; i < 16; ++i)
+                if (kt * 32 + 8 * (i >> 2) + (i & 3) >= lim) s[kt][i] = -INFINITY;
+          }
+          // ---- online softmax, one query per lane (keys split with lane ^ 32)
+          float mx = max3(s[0][0], s[1][0], s[0][1]);
+#pragma unroll
+          for (int i = 1; i < 15; ++i) mx = max3(mx, s[1][i], s[0][i + 1]);
+          mx = fmaxf(mx, s[1][15]);
+          mx = half_max(mx);
+          const bool grow = mx > m_run + p.lag;
+          if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+            const float m_new = grow ? mx : m_run;
+            const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * p.c) : 1.f;
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+              for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+            m_run = m_new;
+          }
+          const float mc = (m_run == -INFINITY) ? 0.f : m_run * p.c;
+          float rs = 0.f;
+#pragma unroll
+          for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const float ex = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], p.c, -mc));
+              s[kt][i] = ex;
+              rs += ex;
+            }
+          l_run += rs;
+          // ---- O^T += V^T . P^T
+#pragma unroll
+          for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              u32x4 pw;
+#pragma unroll
+              for (int q4 = 0; q4 < 4; ++q4) pw[q4] = E::pack2(s[kt][8 * j + 2 * q4], s[kt][8 * j + 2 * q4 + 1]);
+              const short8v pb = __builtin_bit_cast(short8v, pw);
+              const uint32_t vrow = vt_base + (kt * 32 + 16 * j) * RB;
+#pragma unroll
+              for (int dt = 0; dt < DT; ++dt) {
+                const uint32_t a = vrow + (uint32_t)(v_rd ^ (dt * 64));
+                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(uintptr_t)a);
+                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(uintptr_t)(a + 8 * RB));
+                const short8v va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                o[dt] = E::mfma(va, pb, o[dt]);
+              }
+            }
+        }
+        buf ^= 1;
       }
-      // ---- edge tiles: ragged run tail and the causal diagonal
-      const bool edge = valid < kTileKeys || (p.causal && kpos + valid - 1 > wave_kvis_min);
-      if (edge) {
-        int lim = valid;
-        if (p.causal) lim = min(lim, lane_kvis - kpos + 1);
-        lim -= 4 * g32;
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i)
-            if (kt * 32 + 8 * (i >> 2) + (i & 3) >= lim) s[kt][i] = -INFINITY;
+      chunk_base += n;
+      if (chunk_base >= total) break;
+      // a longer item: expand the next chunk of its tile list in place
+      __syncthreads();
+      if (wave == 0) {
+        // (the staged records now belong to a later item, so this item's are fetched again)
+        const int qb = hdr_word(c, H_QB);
+        const QBlockInfo inf = p.info[qb];
+        const uint32_t *row = p.bits + ((size_t)cur_hk * p.nqb + qb) * p.wpr;
+        const int nwords = 2 * ((inf.nkblk + 63) >> 6);
+        (void)build_tile_list(lds_list + c * kListCap, chunk_base, row, nwords, p.kbs, inf.kmax,
+                              lane < nwords ? row[lane] : 0u, lane);
       }
-      // ---- online softmax, one query per lane (keys split with lane ^ 32)
-      float mx = fmaxf(s[0][0], s[1][0]);
-#pragma unroll
-      for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s[0][i], s[1][i]));
-      mx = half_max(mx);
-      const bool grow = mx > m_run + p.lag;
-      if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-        const float m_new = grow ? mx : m_run;
-        const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * p.c) : 1.f;
-        l_run *= alpha;
+      __syncthreads();
+      {   // nothing is in flight here: fetch the chunk's first tile
+        const int e = __builtin_amdgcn_readfirstlane(lds_list[c * kListCap]);
+        const int64_t tok = (e >> 6) << 4;
+        issue_loads(buf, kg + tok * p.k_s, vg + tok * p.v_s, (e & 63) + 1);
+      }
+    }
+
+    // ---- epilogue: normalise, convert, store (rows with no visible key store exact zeros)
+    if (active) {
+      const float l_tot = half_sum(l_run);
+      const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+      if (l32 < nrows) {
+        char *orow = p.out + (int64_t)(row_begin + row0 + l32) * p.o_s + (int64_t)hq * p.o_h;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
-        m_run = m_new;
-      }
-      const float mc = (m_run == -INFINITY) ? 0.f : m_run * p.c;
-      float rs = 0.f;
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], p.c, -mc));
-          s[kt][i] = e;
-          rs += e;
-        }
-      l_run += rs;
-      // ---- O^T += V^T . P^T
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          u32x4 pw;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) pw[e] = E::pack2(s[kt][8 * j + 2 * e], s[kt][8 * j + 2 * e + 1]);
-          const short8v pb = __builtin_bit_cast(short8v, pw);
-          const uint32_t vrow = vt_base + (kt * 32 + 16 * j) * RB;
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) {
-            const uint32_t a = vrow + (uint32_t)(v_rd ^ (dt * 64));
-            const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(uintptr_t)a);
-            const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(uintptr_t)(a + 8 * RB));
-            const short8v va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            o[dt] = E::mfma(va, pb, o[dt]);
+          for (int i4 = 0; i4 < 4; ++i4) {
+            uint2 w;
+            w.x = E::pack2(o[dt][4 * i4 + 0] * inv, o[dt][4 * i4 + 1] * inv);
+            w.y = E::pack2(o[dt][4 * i4 + 2] * inv, o[dt][4 * i4 + 3] * inv);
+            *(uint2 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 2) = w;
           }
-        }
+      }
     }
 
-    if (!have_next) break;
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): next tile has landed
-    __syncthreads();                     // and every wave is done with the current buffers
-    buf ^= 1;
-    kpos = nkpos;
-    valid = nvalid;
-  }
-
-  // ---- epilogue: normalise, convert, store (rows with no visible key store exact zeros)
-  if (active) {
-    const float l_tot = half_sum(l_run);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    if (l32 < nrows) {
-      char *orow = p.out + (int64_t)(info.row_begin + row0 + l32) * p.o_s + (int64_t)hq * p.o_h;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          uint2 w;
-          w.x = E::pack2(o[dt][4 * i4 + 0] * inv, o[dt][4 * i4 + 1] * inv);
-          w.y = E::pack2(o[dt][4 * i4 + 2] * inv, o[dt][4 * i4 + 3] * inv);
-          *(uint2 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 2) = w;
+    // ---- move on to the next item
+    if (total == 0) {
+      // No tile, hence no barrier since this item began: the next list may still be being written,
+      // and nothing of the next item has been requested yet.
+      __syncthreads();
+      nxt_hk = hdr_word(c ^ 1, H_HK);
+      if (nxt_hk >= 0) {
+        if (hdr_word(c ^ 1, H_TOTAL) > 0) {
+          const int e1 = __builtin_amdgcn_readfirstlane(lds_list[(c ^ 1) * kListCap]);
+          const int64_t tok = hdr_word(c ^ 1, H_KEY_BEGIN) + ((e1 >> 6) << 4);
+          issue_loads(buf, p.k + (int64_t)nxt_hk * p.k_h + tok * p.k_s, p.v + (int64_t)nxt_hk * p.v_h + tok * p.v_s,
+                      (e1 & 63) + 1);
         }
+        bool act; int hq1, r01, nr1;
+        const char *qrow = q_row_ptr(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS), act,
+                                     hq1, r01, nr1);
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          u32x4 raw = {0u, 0u, 0u, 0u};
+          if (act) raw = *(const u32x4 *)(qrow + ks * 32);
+          raw ^= p.q_sign;
+          qf[ks] = __builtin_bit_cast(short8v, raw);
+        }
+      }
+      __syncthreads();   // wave 0 rewrites this item's list next; every wave has read its header by now
     }
+    if (nxt_hk < 0) break;
+    c ^= 1;
   }
 }
 
@@ -449,17 +720,33 @@ int fail(int code, const char *fmt, ...) {
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 inline int words_per_row(int num_k_block) { return 2 * ((num_k_block + 63) / 64); }
+// workspace layout: QBlockInfo[num_q_block] | Sched | bit words
+inline size_t sched_offset(int num_q_block) { return align_up((size_t)num_q_block * sizeof(QBlockInfo), 256); }
+inline size_t bits_offset(int num_q_block) { return sched_offset(num_q_block) + align_up(sizeof(Sched), 256); }
+
+int persistent_grid(const void *kernel, int lds_bytes) {
+  int dev = 0, cus = 0, per_cu = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, lds_bytes) != hipSuccess) return 0;
+  if (per_cu < 1) return 0;
+  if (per_cu > 4) per_cu = 4;
+  return cus * per_cu;
+}
 
 template <int D, typename E>
-int launch_fwd(const FwdParams &fp, int grid, hipStream_t stream) {
-  constexpr int lds_bytes = 4 * kTileKeys * D * 2;
-  static thread_local bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
+  constexpr int lds_bytes = 4 * kTileKeys * D * 2 + 2 * H_WORDS * 4 + 2 * kListCap * 4;
+  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E>);
+  static thread_local int resident = 0;   // workgroups that fit the device at once
+  if (resident == 0) {
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_set = true;
+    resident = persistent_grid(kernel, lds_bytes);
+    if (resident <= 0) return fail(HBSA_ERR_UNSUPPORTED, "could not size the persistent grid");
   }
+  const int grid = (int)(items < resident ? items : resident);
+  hipLaunchKernelGGL(hbsa_reset_kernel, dim3(1), dim3(64), 0, stream, fp.sched);
   hipLaunchKernelGGL((hbsa_fwd_kernel<D, E>), dim3(grid), dim3(kThreads), lds_bytes, stream, fp);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail((int)e, "hbsa_fwd_kernel launch: %s", hipGetErrorString(e));
@@ -476,9 +763,8 @@ const char *hbsa_last_error(void) { return g_err; }
 
 size_t hbsa_fwd_workspace_bytes(int32_t nhead_k, int32_t num_q_block, int32_t num_k_block) {
   if (nhead_k <= 0 || num_q_block <= 0 || num_k_block <= 0) return 256;
-  const size_t info = align_up((size_t)num_q_block * sizeof(QBlockInfo), 256);
   const size_t bits = align_up((size_t)nhead_k * num_q_block * words_per_row(num_k_block) * sizeof(uint32_t), 256);
-  return info + bits;
+  return bits_offset(num_q_block) + bits;
 }
 
 int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens, const uint8_t *block_mask,
@@ -508,7 +794,7 @@ int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens, c
   pp.cu_num_q_block = cu_num_q_block; pp.cu_num_k_block = cu_num_k_block;
   pp.mask = block_mask; pp.ms_h = mask_strides[0]; pp.ms_q = mask_strides[1]; pp.ms_k = mask_strides[2];
   pp.info = (QBlockInfo *)workspace;
-  pp.bits = (uint32_t *)((char *)workspace + align_up((size_t)num_q_block * sizeof(QBlockInfo), 256));
+  pp.bits = (uint32_t *)((char *)workspace + bits_offset(num_q_block));
   pp.nqb = num_q_block; pp.qbs = q_block_size; pp.kbs = k_block_size; pp.wpr = words_per_row(num_k_block);
   pp.causal = causal ? 1 : 0;
   hipLaunchKernelGGL(hbsa_prep_kernel, dim3((num_q_block + 3) / 4, nhead_k), dim3(kThreads), 0, (hipStream_t)stream, pp);
@@ -517,7 +803,7 @@ int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens, c
   return 0;
 }
 
-int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out, const void *workspace, size_t workspace_bytes,
+int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out, void *workspace, size_t workspace_bytes,
                  int32_t dtype, int32_t total_q, int32_t total_k, int32_t nhead_q, int32_t nhead_k, int32_t headdim,
                  int32_t num_q_block, int32_t num_k_block, int32_t q_block_size, int32_t k_block_size, int32_t causal,
                  float softmax_scale, const int64_t *strides, void *stream) {
@@ -550,7 +836,9 @@ int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out, const v
   FwdParams fp;
   fp.q = (const char *)q; fp.k = (const char *)k; fp.v = (const char *)v; fp.out = (char *)out;
   fp.info = (const QBlockInfo *)workspace;
-  fp.bits = (const uint32_t *)((const char *)workspace + align_up((size_t)num_q_block * sizeof(QBlockInfo), 256));
+  fp.bits = (const uint32_t *)((const char *)workspace + bits_offset(num_q_block));
+  fp.sched = (Sched *)((char *)workspace + sched_offset(num_q_block));
+  fp.nhead_k = nhead_k;
   fp.q_s = strides[0] * 2; fp.q_h = strides[1] * 2; fp.k_s = strides[2] * 2; fp.k_h = strides[3] * 2;
   fp.v_s = strides[4] * 2; fp.v_h = strides[5] * 2; fp.o_s = strides[6] * 2; fp.o_h = strides[7] * 2;
   fp.nqb = num_q_block; fp.ratio = nhead_q / nhead_k; fp.kbs = k_block_size; fp.wpr = words_per_row(num_k_block);
@@ -562,15 +850,15 @@ int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out, const v
   if (c < 1e-30f) c = 1e-30f;  // scale 0: uniform weights over the visible keys, and -inf * c stays -inf
   fp.c = c;
   fp.lag = kLazyRescaleLog2 / c;
-  const long long grid = (long long)nhead_k * num_q_block * fp.nsub;
-  if (grid > 0x7fffffffLL) return fail(HBSA_ERR_UNSUPPORTED, "too many work items (%lld)", grid);
+  const long long items = (long long)nhead_k * num_q_block * fp.nsub;
+  if (items > 0x7fffffffLL) return fail(HBSA_ERR_UNSUPPORTED, "too many work items (%lld)", items);
 
   hipStream_t st = (hipStream_t)stream;
   const bool bf = dtype == HBSA_DTYPE_BF16;
   switch (headdim) {
-    case 32: return bf ? launch_fwd<32, ElemBF16>(fp, (int)grid, st) : launch_fwd<32, ElemF16>(fp, (int)grid, st);
-    case 64: return bf ? launch_fwd<64, ElemBF16>(fp, (int)grid, st) : launch_fwd<64, ElemF16>(fp, (int)grid, st);
-    default: return bf ? launch_fwd<128, ElemBF16>(fp, (int)grid, st) : launch_fwd<128, ElemF16>(fp, (int)grid, st);
+    case 32: return bf ? launch_fwd<32, ElemBF16>(fp, items, st) : launch_fwd<32, ElemF16>(fp, items, st);
+    case 64: return bf ? launch_fwd<64, ElemBF16>(fp, items, st) : launch_fwd<64, ElemF16>(fp, items, st);
+    default: return bf ? launch_fwd<128, ElemBF16>(fp, items, st) : launch_fwd<128, ElemF16>(fp, items, st);
   }
 }
 

@@ -101,6 +101,8 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out,
  *
  * hbsa_fwd_run runs the attention kernel from a prepared `workspace` (same sizes, block
  * sizes and `causal` as the prepare call; q/k/v/out and softmax_scale may differ per call).
+ * It rewrites the scheduler counters inside `workspace`, so two runs that share one
+ * workspace must be ordered on one stream, not concurrent.
  * It replaces the reference `_fwd_kernel` launch (reference
  * hbsattn/fwd_triton_auto_tile_size.py:283-308).
  *   strides       int64[8] = { q_tok, q_head, k_tok, k_head, v_tok, v_head, out_tok, out_head }
@@ -115,7 +117,7 @@ int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens,
                      const int64_t *mask_strides, void *stream);
 
 int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out,
-                 const void *workspace, size_t workspace_bytes,
+                 void *workspace, size_t workspace_bytes,
                  int32_t dtype, int32_t total_q, int32_t total_k,
                  int32_t nhead_q, int32_t nhead_k, int32_t headdim,
                  int32_t num_q_block, int32_t num_k_block,
