@@ -44,6 +44,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 #define HBSA_AS1(p) ((const __attribute__((address_space(1))) void *)(p))
 #define HBSA_AS3(p) ((__attribute__((address_space(3))) void *)(p))
@@ -225,45 +226,53 @@ __device__ __forceinline__ int build_tile_list(int *list, int chunk_base, const 
   if (kmax <= 0 || nwords <= 0) return 0;
   int total = 0;
   if ((kbs & 63) == 0) {
-    // Blocks are whole tiles: every kept block yields kbs/64 tiles, the one holding key
-    // kmax-1 possibly fewer.  Lane i expands word i; offsets come from a wavefront scan.
+    // Blocks are whole tiles: every kept block yields kbs/64 tiles (those starting at or past
+    // kmax are dropped; they would be the last of the list).  Two bit words are expanded per
+    // step: lane l looks at bit (l & 31) of word 2*step + (l >> 5), and its tiles go right after
+    // the tiles of the kept blocks below it.
     const int tpb = kbs >> 6;
-    const int j_last = (kmax - 1) / kbs;
-    const int t_last = (kmax - j_last * kbs + 63) >> 6;
-    for (int win = 0; win * 64 < nwords; ++win) {
-      const int widx = win * 64 + lane;
-      uint32_t w = win == 0 ? (lane < nwords ? first_words : 0u) : (widx < nwords ? row[widx] : 0u);
-      int cnt = __builtin_popcount(w) * tpb;
-      if ((j_last >> 5) == widx && ((w >> (j_last & 31)) & 1u)) cnt -= tpb - t_last;
-      int incl = cnt;
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const int up = __shfl_up(incl, d);
-        if (lane >= d) incl += up;
+    const int half = lane >> 5, bit = lane & 31;
+    const int j_last = (kmax - 1) / kbs;   // no bit above this block is set
+    int window = 0;
+    uint32_t held = lane < nwords ? first_words : 0u;
+    for (int w2 = 0; w2 < nwords; w2 += 2) {
+      if ((w2 >> 6) != window) {   // rows longer than 2048 blocks only
+        window = w2 >> 6;
+        const int i = window * 64 + lane;
+        held = i < nwords ? row[i] : 0u;
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // wait here, not (for everything in flight) on the common path
+        asm volatile("" : "+v"(held));
       }
-      int off = total + incl - cnt - chunk_base;
-      while (w) {
-        const int j = widx * 32 + __builtin_ctz(w);
-        w &= w - 1;
-        for (int t = 0; t < tpb; ++t) {
+      const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)held, w2 & 63);
+      const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)held, (w2 + 1) & 63);   // nwords is even
+      if ((lo | hi) == 0) continue;
+      const uint32_t mine = half ? hi : lo;
+      if ((mine >> bit) & 1u) {
+        const int below = __builtin_popcount(mine & ((1u << bit) - 1u)) + (half ? __builtin_popcount(lo) : 0);
+        const int j = (w2 + half) * 32 + bit;
+        int off = total + below * tpb - chunk_base;
+        for (int t = 0; t < tpb; ++t, ++off) {
           const int pos = j * kbs + 64 * t;
-          if (pos < kmax) {
-            if (off >= 0 && off < kListCap) list[off] = pack_tile(pos, min(kTileKeys, kmax - pos));
-            ++off;
-          }
+          if (pos < kmax && off >= 0 && off < kListCap) list[off] = pack_tile(pos, min(kTileKeys, kmax - pos));
         }
       }
-      total += __builtin_amdgcn_readlane(incl, 63);
+      total += (__builtin_popcount(lo) + __builtin_popcount(hi)) * tpb;
+      if ((j_last >> 6) == (w2 >> 1)) {   // tiles dropped at the end of the last visible block
+        const uint32_t wsel = (j_last & 32) ? hi : lo;
+        if ((wsel >> (j_last & 31)) & 1u) total -= tpb - ((kmax - j_last * kbs + 63) >> 6);
+      }
     }
   } else {
     // General block sizes: walk the runs of adjacent kept blocks serially (wavefront-uniform).
     int window = 0;
     uint32_t held = lane < nwords ? first_words : 0u;
     auto word = [&](int w) -> uint32_t {
-      if ((w >> 6) != window) {
+      if ((w >> 6) != window) {   // rows longer than 2048 blocks only
         window = w >> 6;
         const int i = window * 64 + lane;
         held = i < nwords ? row[i] : 0u;
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        asm volatile("" : "+v"(held));
       }
       return (uint32_t)__builtin_amdgcn_readlane((int)held, w & 63);
     };
@@ -355,6 +364,8 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
       if (++tries >= 8) break;
       uint32_t r = 0;
       if (lane == 0) r = atomicAdd(&p.sched->qnext[(first_queue + tries) & 7], 1u);
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // only at the tail of the kernel, when a queue has run dry
+      asm volatile("" : "+v"(r));
       claimed = (uint32_t)__builtin_amdgcn_readfirstlane((int)r);
     }
     if (st_hk >= 0) {
@@ -522,6 +533,9 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         const int kpos = (e >> 6) << 4, valid = (e & 63) + 1;
 
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the current tile has landed in LDS
+        // Everything fetched so far has arrived, the scheduler's records included: tell the
+        // compiler here, or it waits for ALL outstanding memory traffic where they are first read.
+        asm volatile("" : "+v"(st_info), "+v"(st_bits), "+v"(pending));
         __syncthreads();                     // ... for every wave, and the other buffers are free
 
         const bool last = chunk_base + t + 1 == total;
@@ -669,10 +683,10 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
           for (int i4 = 0; i4 < 4; ++i4) {
-            uint2 w;
+            u32x2 w;
             w.x = E::pack2(o[dt][4 * i4 + 0] * inv, o[dt][4 * i4 + 1] * inv);
             w.y = E::pack2(o[dt][4 * i4 + 2] * inv, o[dt][4 * i4 + 3] * inv);
-            *(uint2 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 2) = w;
+            *(u32x2 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 2) = w;
           }
       }
     }
@@ -681,6 +695,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     if (total == 0) {
       // No tile, hence no barrier since this item began: the next list may still be being written,
       // and nothing of the next item has been requested yet.
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // keeps "every fetch has arrived" true on every path
       __syncthreads();
       nxt_hk = hdr_word(c ^ 1, H_HK);
       if (nxt_hk >= 0) {
