@@ -31,6 +31,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <type_traits>
 
 #include "hbsattn_amd.h"
 
@@ -306,6 +307,42 @@ __device__ __forceinline__ int build_tile_list(int *list, int chunk_base, const 
   return total;
 }
 
+
+// ---- LDS reads issued by hand.  The compiler neither waits for these nor knows they touch LDS,
+// so each result must pass through lds_wait<N>() before it is used: LDS operations of a
+// wavefront complete in order, and lds_wait<N> returns once at most N of them are outstanding.
+// (The transposing read is issued this way because the compiler otherwise waits for every
+// outstanding global->LDS load before it; the K reads so that their issue distance is fixed.)
+template <int OFF>
+__device__ __forceinline__ short8v lds_read_b128(uint32_t addr) {
+  short8v r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int OFF>
+__device__ __forceinline__ short4v lds_read_tr16_b64(uint32_t addr) {
+  short4v r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=&v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int N>
+__device__ __forceinline__ void lds_wait(short8v &a, short8v &b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void lds_wait(short4v &a, short4v &b, short4v &c, short4v &d, short4v &e, short4v &f, short4v &g,
+                                         short4v &h) {
+  asm volatile("s_waitcnt lgkmcnt(%8)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f), "+v"(g), "+v"(h) : "n"(N));
+}
+
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
 template <int D, typename E>
 __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   constexpr int RB = D * 2;            // row bytes
@@ -563,17 +600,27 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         f32x16 s[2];
         if (compute) {
           const uint32_t kt_base = (uint32_t)(uintptr_t)HBSA_AS3(lds_k + buf * TILE_BYTES);
-          // ---- S^T = K . Q^T  (two 32-key sub-tiles)
+          // ---- S^T = K . Q^T  (two 32-key sub-tiles).  The K operand reads run up to four k-steps
+          // ahead of the MFMAs; every MFMA pair waits only for its own two operands.
 #pragma unroll
           for (int i = 0; i < 16; ++i) { s[0][i] = 0.f; s[1][i] = 0.f; }
-#pragma unroll
-          for (int ks = 0; ks < KSTEPS; ++ks) {
+          constexpr int PF = KSTEPS < 4 ? KSTEPS : 4;   // k-steps whose operands are in flight
+          short8v kb[PF][2];
+          auto read_kstep = [&](auto ks_) {
+            constexpr int ks = decltype(ks_)::value;
             const uint32_t a = kt_base + (uint32_t)(k_rd ^ (ks * 32));
-            const short8v a0 = *(const __attribute__((address_space(3))) short8v *)(uintptr_t)a;
-            const short8v a1 = *(const __attribute__((address_space(3))) short8v *)(uintptr_t)(a + 32 * RB);
-            s[0] = E::mfma(a0, qf[ks], s[0]);
-            s[1] = E::mfma(a1, qf[ks], s[1]);
-          }
+            kb[ks % PF][0] = lds_read_b128<0>(a);
+            kb[ks % PF][1] = lds_read_b128<32 * RB>(a);
+          };
+          static_for<0, PF>(read_kstep);
+          static_for<0, KSTEPS>([&](auto ks_) {
+            constexpr int ks = decltype(ks_)::value;
+            constexpr int ahead = (KSTEPS - 1 - ks) < (PF - 1) ? (KSTEPS - 1 - ks) : (PF - 1);   // k-steps issued after this one
+            lds_wait<2 * ahead>(kb[ks % PF][0], kb[ks % PF][1]);
+            s[0] = E::mfma(kb[ks % PF][0], qf[ks], s[0]);
+            s[1] = E::mfma(kb[ks % PF][1], qf[ks], s[1]);
+            if constexpr (ks + PF < KSTEPS) read_kstep(std::integral_constant<int, ks + PF>{});
+          });
         }
         if (last && nxt_hk >= 0) {
           // Q of this item is no longer needed: fetch the next item's rows under this tile's softmax
@@ -630,25 +677,41 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
               rs += ex;
             }
           l_run += rs;
-          // ---- O^T += V^T . P^T
+          // ---- O^T += V^T . P^T in four groups of 16 keys; the V^T operands of a group are read
+          // while the MFMAs of the group before it run.
+          short4v vb[2][2 * DT];
+          auto read_group = [&](auto g_, short4v *dst) {
+            constexpr int g = decltype(g_)::value;
+            static_for<0, DT>([&](auto dt_) {
+              constexpr int dt = decltype(dt_)::value;
+              const uint32_t a = vt_base + (uint32_t)(v_rd ^ (dt * 64));
+              dst[2 * dt] = lds_read_tr16_b64<g * 16 * RB>(a);
+              dst[2 * dt + 1] = lds_read_tr16_b64<g * 16 * RB + 8 * RB>(a);
+            });
+          };
+          read_group(std::integral_constant<int, 0>{}, vb[0]);
+          static_for<0, 4>([&](auto g_) {
+            constexpr int g = decltype(g_)::value;   // keys 16*g .. 16*g+15 of the tile: kt = g / 2, j = g % 2
+            if constexpr (g + 1 < 4) read_group(std::integral_constant<int, g + 1>{}, vb[(g + 1) & 1]);
+            u32x4 pw;
 #pragma unroll
-          for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              u32x4 pw;
-#pragma unroll
-              for (int q4 = 0; q4 < 4; ++q4) pw[q4] = E::pack2(s[kt][8 * j + 2 * q4], s[kt][8 * j + 2 * q4 + 1]);
-              const short8v pb = __builtin_bit_cast(short8v, pw);
-              const uint32_t vrow = vt_base + (kt * 32 + 16 * j) * RB;
-#pragma unroll
-              for (int dt = 0; dt < DT; ++dt) {
-                const uint32_t a = vrow + (uint32_t)(v_rd ^ (dt * 64));
-                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(uintptr_t)a);
-                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(uintptr_t)(a + 8 * RB));
-                const short8v va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                o[dt] = E::mfma(va, pb, o[dt]);
-              }
+            for (int q4 = 0; q4 < 4; ++q4)
+              pw[q4] = E::pack2(s[g / 2][8 * (g % 2) + 2 * q4], s[g / 2][8 * (g % 2) + 2 * q4 + 1]);
+            const short8v pb = __builtin_bit_cast(short8v, pw);
+            short4v *v = vb[g & 1];
+            if constexpr (DT == 4) {
+              lds_wait<(g + 1 < 4) ? 8 : 0>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]);
+            } else if constexpr (DT == 2) {
+              asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : "n"((g + 1 < 4) ? 4 : 0));
+            } else {
+              asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(v[0]), "+v"(v[1]) : "n"((g + 1 < 4) ? 2 : 0));
             }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+              const short8v va = __builtin_shufflevector(v[2 * dt], v[2 * dt + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+              o[dt] = E::mfma(va, pb, o[dt]);
+            }
+          });
         }
         buf ^= 1;
       }
