@@ -142,6 +142,11 @@ struct ElemBF16 {
     bf16x2 v = {(__bf16)lo, (__bf16)hi};
     return __builtin_bit_cast(uint32_t, v);
   }
+  // acc + lo + hi of a packed pair (v_dot2c_f32_bf16 with a vector of ones)
+  static __device__ __forceinline__ float dot2_ones(uint32_t packed, float acc) {
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, packed), ones, acc, false);
+  }
 };
 struct ElemF16 {
   static __device__ __forceinline__ f32x16 mfma(short8v a, short8v b, f32x16 c) {
@@ -150,6 +155,10 @@ struct ElemF16 {
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     f16x2 v = {(_Float16)lo, (_Float16)hi};
     return __builtin_bit_cast(uint32_t, v);
+  }
+  static __device__ __forceinline__ float dot2_ones(uint32_t packed, float acc) {
+    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, packed), ones, acc, false);
   }
 };
 
@@ -324,6 +333,10 @@ __device__ __forceinline__ short4v lds_read_tr16_b64(uint32_t addr) {
   short4v r;
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=&v"(r) : "v"(addr), "n"(OFF));
   return r;
+}
+template <int N>
+__device__ __forceinline__ void lds_wait1(short8v &a) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N));
 }
 template <int N>
 __device__ __forceinline__ void lds_wait(short8v &a, short8v &b) {
@@ -597,90 +610,78 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         }
 
         const bool compute = active && (!p.causal || kpos <= wave_kvis_max);
-        f32x16 s[2];
         if (compute) {
+          // The tile is processed as two halves of 32 keys so that, inside one wavefront, the
+          // matrix cores always have work queued while the vector ALU does the softmax of the
+          // other half:   S0, max(S0) | S1 + exp(S0) | PV0 + max(S1), exp(S1) | PV1.
           const uint32_t kt_base = (uint32_t)(uintptr_t)HBSA_AS3(lds_k + buf * TILE_BYTES);
-          // ---- S^T = K . Q^T  (two 32-key sub-tiles).  The K operand reads run up to four k-steps
-          // ahead of the MFMAs; every MFMA pair waits only for its own two operands.
+          const uint32_t vt_base = (uint32_t)(uintptr_t)HBSA_AS3(lds_v + buf * TILE_BYTES);
+          const bool edge = valid < kTileKeys || (p.causal && kpos + valid - 1 > wave_kvis_min);
+          int lim = valid;                      // keys (of this lane's query) below lim are visible
+          if (p.causal) lim = min(lim, lane_kvis - kpos + 1);
+          lim -= 4 * g32;
+
+          f32x16 s0, s1;
 #pragma unroll
-          for (int i = 0; i < 16; ++i) { s[0][i] = 0.f; s[1][i] = 0.f; }
-          constexpr int PF = KSTEPS < 4 ? KSTEPS : 4;   // k-steps whose operands are in flight
-          short8v kb[PF][2];
-          auto read_kstep = [&](auto ks_) {
-            constexpr int ks = decltype(ks_)::value;
-            const uint32_t a = kt_base + (uint32_t)(k_rd ^ (ks * 32));
-            kb[ks % PF][0] = lds_read_b128<0>(a);
-            kb[ks % PF][1] = lds_read_b128<32 * RB>(a);
-          };
-          static_for<0, PF>(read_kstep);
+          for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
+
+          // ---- S0 = K[0:32] . Q^T ; the operand reads of S1 are issued as S0 frees the registers
+          short8v kb[KSTEPS];
           static_for<0, KSTEPS>([&](auto ks_) {
             constexpr int ks = decltype(ks_)::value;
-            constexpr int ahead = (KSTEPS - 1 - ks) < (PF - 1) ? (KSTEPS - 1 - ks) : (PF - 1);   // k-steps issued after this one
-            lds_wait<2 * ahead>(kb[ks % PF][0], kb[ks % PF][1]);
-            s[0] = E::mfma(kb[ks % PF][0], qf[ks], s[0]);
-            s[1] = E::mfma(kb[ks % PF][1], qf[ks], s[1]);
-            if constexpr (ks + PF < KSTEPS) read_kstep(std::integral_constant<int, ks + PF>{});
+            kb[ks] = lds_read_b128<0>(kt_base + (uint32_t)(k_rd ^ (ks * 32)));
           });
-        }
-        if (last && nxt_hk >= 0) {
-          // Q of this item is no longer needed: fetch the next item's rows under this tile's softmax
-          bool act; int hq1, r01, nr1;
-          const char *qrow = q_row_ptr(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS),
-                                       act, hq1, r01, nr1);
-#pragma unroll
-          for (int ks = 0; ks < KSTEPS; ++ks) {
-            u32x4 raw = {0u, 0u, 0u, 0u};
-            if (act) raw = *(const u32x4 *)(qrow + ks * 32);
-            raw ^= p.q_sign;
-            qf[ks] = __builtin_bit_cast(short8v, raw);
-          }
-        }
-        if (compute) {
-          const uint32_t vt_base = (uint32_t)(uintptr_t)HBSA_AS3(lds_v + buf * TILE_BYTES);
-          // ---- edge tiles: ragged run tail and the causal diagonal
-          const bool edge = valid < kTileKeys || (p.causal && kpos + valid - 1 > wave_kvis_min);
-          if (edge) {
-            int lim = valid;
-            if (p.causal) lim = min(lim, lane_kvis - kpos + 1);
-            lim -= 4 * g32;
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
+          static_for<0, KSTEPS>([&](auto ks_) {
+            constexpr int ks = decltype(ks_)::value;
+            lds_wait1<KSTEPS - 1>(kb[ks]);
+            s0 = E::mfma(kb[ks], qf[ks], s0);
+            kb[ks] = lds_read_b128<32 * RB>(kt_base + (uint32_t)(k_rd ^ (ks * 32)));
+          });
+
+          // row max of one half, merged into the running max; O and l are rescaled (rarely:
+          // the running max may lag the true one by 2^kLazyRescaleLog2)
+          auto half_rowmax = [&](f32x16 &sh, int key0) {
+            if (edge) {
 #pragma unroll
               for (int i = 0; i < 16; ++i)
-                if (kt * 32 + 8 * (i >> 2) + (i & 3) >= lim) s[kt][i] = -INFINITY;
-          }
-          // ---- online softmax, one query per lane (keys split with lane ^ 32)
-          float mx = max3(s[0][0], s[1][0], s[0][1]);
-#pragma unroll
-          for (int i = 1; i < 15; ++i) mx = max3(mx, s[1][i], s[0][i + 1]);
-          mx = fmaxf(mx, s[1][15]);
-          mx = half_max(mx);
-          const bool grow = mx > m_run + p.lag;
-          if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-            const float m_new = grow ? mx : m_run;
-            const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * p.c) : 1.f;
-            l_run *= alpha;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-              for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
-            m_run = m_new;
-          }
-          const float mc = (m_run == -INFINITY) ? 0.f : m_run * p.c;
-          float rs = 0.f;
-#pragma unroll
-          for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const float ex = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], p.c, -mc));
-              s[kt][i] = ex;
-              rs += ex;
+                if (key0 + 8 * (i >> 2) + (i & 3) >= lim) sh[i] = -INFINITY;
             }
-          l_run += rs;
-          // ---- O^T += V^T . P^T in four groups of 16 keys; the V^T operands of a group are read
-          // while the MFMAs of the group before it run.
-          short4v vb[2][2 * DT];
-          auto read_group = [&](auto g_, short4v *dst) {
+            // The first reduction step is an instruction the compiler knows, so that it inserts
+            // the wait states an MFMA result needs before the vector ALU may read it; the
+            // hand-written v_max3 steps all depend on that first result.
+            float mx = __builtin_amdgcn_fmed3f(sh[0], sh[1], INFINITY);   // = max(sh[0], sh[1])
+#pragma unroll
+            for (int i = 2; i < 16; i += 2) mx = max3(mx, sh[i], sh[i + 1]);
+            mx = half_max(mx);
+            const bool grow = mx > m_run + p.lag;
+            if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+              const float m_new = grow ? mx : m_run;
+              const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * p.c) : 1.f;
+              l_run *= alpha;
+#pragma unroll
+              for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+              m_run = m_new;
+            }
+          };
+          // exponentials of one half, packed to the element type (two groups of 16 keys), row sum
+          auto half_exp = [&](const f32x16 &sh, short8v &p_lo, short8v &p_hi) {
+            const float mc = (m_run == -INFINITY) ? 0.f : m_run * p.c;
+            u32x4 w[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+              for (int q4 = 0; q4 < 4; ++q4) {
+                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sh[8 * j + 2 * q4], p.c, -mc));
+                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sh[8 * j + 2 * q4 + 1], p.c, -mc));
+                w[j][q4] = E::pack2(e0, e1);
+                l_run = E::dot2_ones(w[j][q4], l_run);   // sums what the PV product will actually use
+              }
+            p_lo = __builtin_bit_cast(short8v, w[0]);
+            p_hi = __builtin_bit_cast(short8v, w[1]);
+          };
+          auto read_vgroup = [&](auto g_, short4v *dst) {   // V^T operands of keys 16*g .. 16*g+15
             constexpr int g = decltype(g_)::value;
             static_for<0, DT>([&](auto dt_) {
               constexpr int dt = decltype(dt_)::value;
@@ -689,29 +690,80 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
               dst[2 * dt + 1] = lds_read_tr16_b64<g * 16 * RB + 8 * RB>(a);
             });
           };
-          read_group(std::integral_constant<int, 0>{}, vb[0]);
-          static_for<0, 4>([&](auto g_) {
-            constexpr int g = decltype(g_)::value;   // keys 16*g .. 16*g+15 of the tile: kt = g / 2, j = g % 2
-            if constexpr (g + 1 < 4) read_group(std::integral_constant<int, g + 1>{}, vb[(g + 1) & 1]);
-            u32x4 pw;
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4)
-              pw[q4] = E::pack2(s[g / 2][8 * (g % 2) + 2 * q4], s[g / 2][8 * (g % 2) + 2 * q4 + 1]);
-            const short8v pb = __builtin_bit_cast(short8v, pw);
-            short4v *v = vb[g & 1];
+          auto wait_vgroup = [&](auto n_, short4v *v) {
+            constexpr int n = decltype(n_)::value;
             if constexpr (DT == 4) {
-              lds_wait<(g + 1 < 4) ? 8 : 0>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]);
+              lds_wait<n>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]);
             } else if constexpr (DT == 2) {
-              asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : "n"((g + 1 < 4) ? 4 : 0));
+              asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : "n"(n));
             } else {
-              asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(v[0]), "+v"(v[1]) : "n"((g + 1 < 4) ? 2 : 0));
+              asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(v[0]), "+v"(v[1]) : "n"(n));
             }
+          };
+          auto pv_group = [&](const short8v &pb, const short4v *v) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
               const short8v va = __builtin_shufflevector(v[2 * dt], v[2 * dt + 1], 0, 1, 2, 3, 4, 5, 6, 7);
               o[dt] = E::mfma(va, pb, o[dt]);
             }
+          };
+
+          half_rowmax(s0, 0);
+
+          // ---- S1 = K[32:64] . Q^T   overlapped with   P0 = exp(S0)
+          short8v p0a, p0b, p1a, p1b;
+          static_for<0, KSTEPS>([&](auto ks_) {
+            constexpr int ks = decltype(ks_)::value;
+            lds_wait1<KSTEPS - 1 - ks>(kb[ks]);
+            s1 = E::mfma(kb[ks], qf[ks], s1);
           });
+          short4v vb[2][2 * DT];
+          read_vgroup(std::integral_constant<int, 0>{}, vb[0]);
+          read_vgroup(std::integral_constant<int, 1>{}, vb[1]);
+          half_exp(s0, p0a, p0b);
+
+          if (last && nxt_hk >= 0) {
+            // Q of this item is no longer needed: fetch the next item's rows under the rest of this tile
+            bool act; int hq1, r01, nr1;
+            const char *qrow = q_row_ptr(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS),
+                                         act, hq1, r01, nr1);
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+              u32x4 raw = {0u, 0u, 0u, 0u};
+              if (act) raw = *(const u32x4 *)(qrow + ks * 32);
+              raw ^= p.q_sign;
+              qf[ks] = __builtin_bit_cast(short8v, raw);
+            }
+          }
+
+          // ---- O^T += V^T[:, 0:32] . P0   overlapped with   row max of S1 and P1 = exp(S1).
+          // (P0 was formed under the running max as it stood after S0, so its product has to be
+          // queued before the row max of S1 may rescale O.)
+          wait_vgroup(std::integral_constant<int, 2 * DT>{}, vb[0]);
+          pv_group(p0a, vb[0]);
+          read_vgroup(std::integral_constant<int, 2>{}, vb[0]);
+          wait_vgroup(std::integral_constant<int, 2 * DT>{}, vb[1]);
+          pv_group(p0b, vb[1]);
+          read_vgroup(std::integral_constant<int, 3>{}, vb[1]);
+          half_rowmax(s1, 32);
+          half_exp(s1, p1a, p1b);
+
+          // ---- O^T += V^T[:, 32:64] . P1
+          wait_vgroup(std::integral_constant<int, 2 * DT>{}, vb[0]);
+          pv_group(p1a, vb[0]);
+          wait_vgroup(std::integral_constant<int, 0>{}, vb[1]);
+          pv_group(p1b, vb[1]);
+        } else if (last && nxt_hk >= 0) {
+          bool act; int hq1, r01, nr1;
+          const char *qrow = q_row_ptr(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS), act,
+                                       hq1, r01, nr1);
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            u32x4 raw = {0u, 0u, 0u, 0u};
+            if (act) raw = *(const u32x4 *)(qrow + ks * 32);
+            raw ^= p.q_sign;
+            qf[ks] = __builtin_bit_cast(short8v, raw);
+          }
         }
         buf ^= 1;
       }
