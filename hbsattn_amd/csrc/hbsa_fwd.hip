@@ -142,6 +142,9 @@ struct ElemBF16 {
     bf16x2 v = {(__bf16)lo, (__bf16)hi};
     return __builtin_bit_cast(uint32_t, v);
   }
+  static __device__ __forceinline__ uint32_t scale_packed(uint32_t w, float f) {
+    return pack2(__builtin_bit_cast(float, w << 16) * f, __builtin_bit_cast(float, w & 0xffff0000u) * f);
+  }
   // acc + lo + hi of a packed pair (v_dot2c_f32_bf16 with a vector of ones)
   static __device__ __forceinline__ float dot2_ones(uint32_t packed, float acc) {
     const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
@@ -155,6 +158,10 @@ struct ElemF16 {
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     f16x2 v = {(_Float16)lo, (_Float16)hi};
     return __builtin_bit_cast(uint32_t, v);
+  }
+  static __device__ __forceinline__ uint32_t scale_packed(uint32_t w, float f) {
+    const f16x2 v = __builtin_bit_cast(f16x2, w);
+    return pack2((float)v.x * f, (float)v.y * f);
   }
   static __device__ __forceinline__ float dot2_ones(uint32_t packed, float acc) {
     const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
@@ -212,6 +219,11 @@ struct Sched {
 __global__ void hbsa_reset_kernel(Sched *s) {
   if (threadIdx.x < 8) s->qnext[threadIdx.x] = 0;
 }
+
+#ifndef HBSA_INTERLEAVE_C
+#define HBSA_INTERLEAVE_C
+#define HBSA_INTERLEAVE_D
+#endif
 
 constexpr int kListCap = 1024;   // tile entries per list; longer items are expanded in chunks
 
@@ -468,23 +480,29 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     ld_koff[i] = (uint32_t)r * (uint32_t)p.k_s + (uint32_t)ld_kchunk[i];
     ld_voff[i] = (uint32_t)r * (uint32_t)p.v_s + (uint32_t)ld_vchunk[i];
   }
-  // kbase / vbase: wavefront-uniform address of the tile's first key row (for this kv head)
+  const uint32_t lds_k_addr = (uint32_t)(uintptr_t)HBSA_AS3(lds_k);
+  const uint32_t lds_v_addr = (uint32_t)(uintptr_t)HBSA_AS3(lds_v);
+  // kbase / vbase: wavefront-uniform address of the tile's first key row (for this kv head).
+  // 16 bytes per lane go straight from global memory into LDS at (M0 + 16 * lane); the global
+  // address is a scalar base plus a 32-bit per-lane offset.
+  auto dma16 = [&](const char *sbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(sbase)
+                 : "memory", "m0");
+  };
   auto issue_loads = [&](int buf, const char *kbase, const char *vbase, int valid) {
-    if (valid == kTileKeys) {
 #pragma unroll
-      for (int i = 0; i < LOADS; ++i) {
-        const int lds_off = buf * TILE_BYTES + (i * 4 + wave) * 1024;
-        __builtin_amdgcn_global_load_lds(HBSA_AS1(kbase + ld_koff[i]), HBSA_AS3(lds_k + lds_off), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(HBSA_AS1(vbase + ld_voff[i]), HBSA_AS3(lds_v + lds_off), 16, 0, 0);
-      }
-    } else {   // ragged tail of a run: rows past the end re-read the last valid row (masked later)
-#pragma unroll
-      for (int i = 0; i < LOADS; ++i) {
+    for (int i = 0; i < LOADS; ++i) {
+      uint32_t ko = ld_koff[i], vo = ld_voff[i];
+      if (valid != kTileKeys) {   // ragged tail of a run: rows past the end re-read the last valid row (masked later)
         const uint32_t r = (uint32_t)min(ld_row[i], valid - 1);
-        const int lds_off = buf * TILE_BYTES + (i * 4 + wave) * 1024;
-        __builtin_amdgcn_global_load_lds(HBSA_AS1(kbase + (r * (uint32_t)p.k_s + (uint32_t)ld_kchunk[i])), HBSA_AS3(lds_k + lds_off), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(HBSA_AS1(vbase + (r * (uint32_t)p.v_s + (uint32_t)ld_vchunk[i])), HBSA_AS3(lds_v + lds_off), 16, 0, 0);
+        ko = r * (uint32_t)p.k_s + (uint32_t)ld_kchunk[i];
+        vo = r * (uint32_t)p.v_s + (uint32_t)ld_vchunk[i];
       }
+      const uint32_t lds_off = (uint32_t)(buf * TILE_BYTES + (i * 4 + wave) * 1024);
+      dma16(kbase, ko, lds_k_addr + lds_off);
+      dma16(vbase, vo, lds_v_addr + lds_off);
     }
   };
 
@@ -625,17 +643,26 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 #pragma unroll
           for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
 
-          // ---- S0 = K[0:32] . Q^T ; the operand reads of S1 are issued as S0 frees the registers
-          short8v kb[KSTEPS];
-          static_for<0, KSTEPS>([&](auto ks_) {
-            constexpr int ks = decltype(ks_)::value;
-            kb[ks] = lds_read_b128<0>(kt_base + (uint32_t)(k_rd ^ (ks * 32)));
-          });
-          static_for<0, KSTEPS>([&](auto ks_) {
-            constexpr int ks = decltype(ks_)::value;
-            lds_wait1<KSTEPS - 1>(kb[ks]);
-            s0 = E::mfma(kb[ks], qf[ks], s0);
-            kb[ks] = lds_read_b128<32 * RB>(kt_base + (uint32_t)(k_rd ^ (ks * 32)));
+          // ---- K operand reads: 2 * KSTEPS reads (all k-steps of the first 32 keys, then of the
+          // second 32), PF of them in flight, each consumed by one MFMA
+          constexpr int PF = 4;
+          constexpr int NK = 2 * KSTEPS;
+          short8v kb[PF];
+          auto read_k = [&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            constexpr int ks = i % KSTEPS;
+            const uint32_t a = kt_base + (uint32_t)(k_rd ^ (ks * 32));
+            if constexpr (i < KSTEPS) kb[i % PF] = lds_read_b128<0>(a);
+            else kb[i % PF] = lds_read_b128<32 * RB>(a);
+          };
+          static_for<0, PF>(read_k);
+          // ---- S0 = K[0:32] . Q^T
+          static_for<0, KSTEPS>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            constexpr int ahead = (NK - 1 - i) < (PF - 1) ? (NK - 1 - i) : (PF - 1);
+            lds_wait1<ahead>(kb[i % PF]);
+            s0 = E::mfma(kb[i % PF], qf[i % KSTEPS], s0);
+            if constexpr (i + PF < NK) read_k(std::integral_constant<int, i + PF>{});
           });
 
           // row max of one half, merged into the running max; O and l are rescaled (rarely:
@@ -710,50 +737,73 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 
           half_rowmax(s0, 0);
 
-          // ---- S1 = K[32:64] . Q^T   overlapped with   P0 = exp(S0)
+          // ---- S1 = K[32:64] . Q^T   interleaved with   P0 = exp(S0)
           short8v p0a, p0b, p1a, p1b;
-          static_for<0, KSTEPS>([&](auto ks_) {
-            constexpr int ks = decltype(ks_)::value;
-            lds_wait1<KSTEPS - 1 - ks>(kb[ks]);
-            s1 = E::mfma(kb[ks], qf[ks], s1);
+          static_for<KSTEPS, NK>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            constexpr int ahead = (NK - 1 - i) < (PF - 1) ? (NK - 1 - i) : (PF - 1);
+            lds_wait1<ahead>(kb[i % PF]);
+            s1 = E::mfma(kb[i % PF], qf[i % KSTEPS], s1);
+            if constexpr (i + PF < NK) read_k(std::integral_constant<int, i + PF>{});
           });
           short4v vb[2][2 * DT];
           read_vgroup(std::integral_constant<int, 0>{}, vb[0]);
           read_vgroup(std::integral_constant<int, 1>{}, vb[1]);
           half_exp(s0, p0a, p0b);
+          HBSA_INTERLEAVE_C
 
-          if (last && nxt_hk >= 0) {
-            // Q of this item is no longer needed: fetch the next item's rows under the rest of this tile
-            bool act; int hq1, r01, nr1;
-            const char *qrow = q_row_ptr(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS),
-                                         act, hq1, r01, nr1);
+          // ---- row max of S1.  P0 was formed under the running max as it stood after S0 and is not
+          // accumulated yet, so if that max has to move now (rare), P0 is rescaled along with O and l.
+          {
+            if (edge) {
 #pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) {
-              u32x4 raw = {0u, 0u, 0u, 0u};
-              if (act) raw = *(const u32x4 *)(qrow + ks * 32);
-              raw ^= p.q_sign;
-              qf[ks] = __builtin_bit_cast(short8v, raw);
+              for (int i = 0; i < 16; ++i)
+                if (32 + 8 * (i >> 2) + (i & 3) >= lim) s1[i] = -INFINITY;
+            }
+            float mx = __builtin_amdgcn_fmed3f(s1[0], s1[1], INFINITY);
+#pragma unroll
+            for (int i = 2; i < 16; i += 2) mx = max3(mx, s1[i], s1[i + 1]);
+            mx = half_max(mx);
+            const bool grow = mx > m_run + p.lag;
+            if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+              const float m_new = grow ? mx : m_run;
+              const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * p.c) : 1.f;
+              l_run *= alpha;
+#pragma unroll
+              for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+              u32x4 wa = __builtin_bit_cast(u32x4, p0a), wb = __builtin_bit_cast(u32x4, p0b);
+#pragma unroll
+              for (int q4 = 0; q4 < 4; ++q4) {
+                wa[q4] = E::scale_packed(wa[q4], alpha);
+                wb[q4] = E::scale_packed(wb[q4], alpha);
+              }
+              p0a = __builtin_bit_cast(short8v, wa);
+              p0b = __builtin_bit_cast(short8v, wb);
+              m_run = m_new;
             }
           }
 
-          // ---- O^T += V^T[:, 0:32] . P0   overlapped with   row max of S1 and P1 = exp(S1).
-          // (P0 was formed under the running max as it stood after S0, so its product has to be
-          // queued before the row max of S1 may rescale O.)
+          // ---- O^T += V^T[:, 0:32] . P0   interleaved with   P1 = exp(S1)
           wait_vgroup(std::integral_constant<int, 2 * DT>{}, vb[0]);
           pv_group(p0a, vb[0]);
           read_vgroup(std::integral_constant<int, 2>{}, vb[0]);
           wait_vgroup(std::integral_constant<int, 2 * DT>{}, vb[1]);
           pv_group(p0b, vb[1]);
           read_vgroup(std::integral_constant<int, 3>{}, vb[1]);
-          half_rowmax(s1, 32);
           half_exp(s1, p1a, p1b);
+          HBSA_INTERLEAVE_D
 
           // ---- O^T += V^T[:, 32:64] . P1
           wait_vgroup(std::integral_constant<int, 2 * DT>{}, vb[0]);
           pv_group(p1a, vb[0]);
           wait_vgroup(std::integral_constant<int, 0>{}, vb[1]);
           pv_group(p1b, vb[1]);
-        } else if (last && nxt_hk >= 0) {
+        }
+        if (last && nxt_hk >= 0) {
+          // Q of this item is no longer needed: fetch the next item's rows while the last MFMAs
+          // drain and the epilogue runs
           bool act; int hq1, r01, nr1;
           const char *qrow = q_row_ptr(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS), act,
                                        hq1, r01, nr1);
