@@ -44,6 +44,11 @@ DESCRIPTIONS = {
 # which roof bounds the attention kernel at each workload (arithmetic intensity against the
 # ridge at 2500 TFLOP/s / 8 TB/s = 312 FLOP/B)
 BOUND = {"C2": "hbm", "T": "mfma", "C3": "mfma", "C4": "mfma", "C5": "hbm"}
+# HBM bytes per launch of the attention kernel, from rocprofv3 counter runs of this program
+# (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, scaled by what the same counters read for a
+# 1 GiB device-to-device copy: factors 2.000 and 1.000).  Not measured live: a counter run needs
+# the profiler.  The summaries are under profiles/.
+MEASURED_TRAFFIC_BYTES = {"C2": 4.92e9, "T": 56.8e9}
 
 
 def time_steps(fn, steps, warmup):
@@ -111,12 +116,12 @@ def measure(name, steps, warmup):
     if BOUND[name] == "mfma":
         ach = work["flops"] / kernel_ms / 1e9
         res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                           "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "hbsa_fwd_kernel",
+                           "frac": ach / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": "hbsa_fwd_kernel",
                            "kernel_ms": kernel_ms, "algorithmic_flops": work["flops"]}
     else:
         ach = work["bytes"] / kernel_ms / 1e6
         res["roofline"] = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                           "frac": ach / PEAK_HBM_GBS, "traffic": None, "kernel": "hbsa_fwd_kernel",
+                           "frac": ach / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": "hbsa_fwd_kernel",
                            "kernel_ms": kernel_ms, "algorithmic_bytes": work["bytes"],
                            "mfma_frac": work["flops"] / kernel_ms / 1e9 / PEAK_BF16_TFLOPS}
     return w, res
@@ -168,18 +173,30 @@ def cpu_baseline(w, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2", choices=sorted(DESCRIPTIONS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-target", action="store_true", help="skip the extra measurement at the 32K target shape")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a 1 GiB device-to-device copy K times (the known-size kernel the HBM counters "
+                         "of a profile are scaled by)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; sequences and kv heads shard with no exchange, "
                  "so --gpus N>1 is not measured here (use --gpus 1)")
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+
+    if a.copy_calibration:
+        n = 1 << 30
+        src = torch.full((n // 4,), 1.0, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        ms = time_steps(lambda: dst.copy_(src), a.steps, a.warmup)
+        print(json.dumps({"copy_bytes_read": n, "copy_bytes_written": n, "ms_per_copy": ms,
+                          "GBps": 2 * n / ms / 1e6}))
+        return
 
     w, res = measure(a.workload, a.steps, a.warmup)
     line = {

@@ -9,8 +9,9 @@
  * binding for that launcher would need; each cites the reference code it replaces.
  *
  * Conventions
- *   - every pointer named `*_dev` / tensor pointer is DEVICE memory owned by the
- *     caller; the library never allocates, frees or retains device memory;
+ *   - every pointer argument except `strides` / `mask_strides` (host arrays read during
+ *     the call) is DEVICE memory owned by the caller; the library never allocates,
+ *     frees or retains device memory;
  *   - all launches go to `stream` (a hipStream_t passed as void*; NULL = the null
  *     stream) and the calls return without synchronising;
  *   - return value 0 = success, negative = invalid argument (message available

@@ -242,3 +242,54 @@ def test_calculate_blocks_on_device_matches_cpu():
     assert a[0] == b[0] == 12
     for x, y in zip(a[1:], b[1:]):
         assert y.is_cuda and x.dtype == y.dtype and torch.equal(x, y.cpu())
+
+
+# ---------------------------------------------------------------------------------------
+# the combined C entry point, called the way a foreign binding would
+# ---------------------------------------------------------------------------------------
+def _call_hbsa_fwd(w, workspace_bytes=None, headdim=None):
+    import ctypes
+
+    from hbsattn_amd import _lib
+
+    lib = _lib.load()
+    nqb, _, qb2b, cu_nqb = w.q_meta
+    nkb, _, _, cu_nkb = w.k_meta
+    i32 = lambda t: t.to(torch.int32).contiguous()
+    cu_q, cu_k, qb2b, cu_nqb, cu_nkb = map(i32, (w.cu_q_seqlens, w.cu_k_seqlens, qb2b, cu_nqb, cu_nkb))
+    out = torch.full_like(w.q, float("nan"))
+    need = lib.hbsa_fwd_workspace_bytes(w.k.shape[1], nqb, nkb)
+    ws = torch.empty(need, dtype=torch.uint8, device=w.q.device)
+    strides = (ctypes.c_int64 * 11)(w.q.stride(0), w.q.stride(1), w.k.stride(0), w.k.stride(1), w.v.stride(0),
+                                    w.v.stride(1), out.stride(0), out.stride(1), *w.block_mask.stride())
+    scale = w.softmax_scale if w.softmax_scale is not None else w.q.shape[2] ** -0.5
+    rc = lib.hbsa_fwd(w.q.data_ptr(), w.k.data_ptr(), w.v.data_ptr(), out.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),
+                      w.block_mask.data_ptr(), qb2b.data_ptr(), cu_nqb.data_ptr(), cu_nkb.data_ptr(), ws.data_ptr(),
+                      need if workspace_bytes is None else workspace_bytes,
+                      0 if w.q.dtype == torch.bfloat16 else 1, len(w.cu_q) - 1, w.q.shape[0], w.k.shape[0],
+                      w.q.shape[1], w.k.shape[1], w.q.shape[2] if headdim is None else headdim, nqb, nkb,
+                      w.q_block_size, w.k_block_size, int(w.causal), scale, strides,
+                      torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return rc, out, _lib.last_error()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_combined_c_entry_point_matches_operator_and_oracle(dtype):
+    w = make_problem(seed=21, q_lens=[700, 1300, 64], k_lens=[900, 1300, 200], hq=8, hk=4, d=64, qbs=48, kbs=80, keep=0.4,
+                     diag=True, causal=True, scale=0.2, dtype=dtype)
+    rc, out, _ = _call_hbsa_fwd(w)
+    assert rc == 0
+    assert torch.equal(out, _run(w))
+    assert_close_to_oracle(out, oracle_for(w), "hbsa_fwd")
+
+
+def test_combined_c_entry_point_rejects_bad_arguments_without_launching():
+    w = make_problem(seed=22, q_lens=[256], k_lens=[256], hq=2, hk=2, d=64, qbs=64, kbs=64, keep=0.5, diag=True,
+                     causal=False, scale=None)
+    rc, out, msg = _call_hbsa_fwd(w, workspace_bytes=16)
+    assert rc == -3 and "workspace" in msg
+    assert torch.isnan(out.float()).all()
+    rc, out, msg = _call_hbsa_fwd(w, headdim=48)
+    assert rc == -2 and "headdim" in msg
+    assert torch.isnan(out.float()).all()
