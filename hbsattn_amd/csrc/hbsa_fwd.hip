@@ -380,7 +380,6 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   char *lds_k = lds;
-  char *lds_v = lds + 2 * TILE_BYTES;
   int *lds_hdr = (int *)(lds + 4 * TILE_BYTES);     // [2][H_WORDS]
   int *lds_list = lds_hdr + 2 * H_WORDS;            // [2][kListCap]
 
@@ -467,42 +466,53 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 
   // ------------------------------------------------------------------ per-thread constants
   // tile loads: thread -> (row, 16-byte chunk) of the tile, same for every tile
-  int ld_row[LOADS];
   uint32_t ld_koff[LOADS], ld_voff[LOADS];   // byte offset of the thread's chunk from the tile's first row
-  int ld_kchunk[LOADS], ld_vchunk[LOADS];
+  const uint32_t ks32 = (uint32_t)p.k_s, vs32 = (uint32_t)p.v_s;   // row strides in bytes (the host checks they fit)
+  auto ld_place = [&](int i, int &r, uint32_t &kchunk, uint32_t &vchunk) {
+    const int c = (i * 4 + wave) * 64 + lane;
+    const int pc = c % CPR;
+    r = c / CPR;
+    kchunk = (uint32_t)((pc ^ ((r / RPG) % CPR)) * 16);
+    vchunk = (uint32_t)((pc ^ ((CPR >= 8) ? (((r / RPG) % (CPR / 4)) << 2) : 0)) * 16);
+  };
 #pragma unroll
   for (int i = 0; i < LOADS; ++i) {
-    const int c = (i * 4 + wave) * 64 + lane;
-    const int r = c / CPR, pc = c % CPR;
-    ld_row[i] = r;
-    ld_kchunk[i] = (pc ^ ((r / RPG) % CPR)) * 16;
-    ld_vchunk[i] = (pc ^ ((CPR >= 8) ? (((r / RPG) % (CPR / 4)) << 2) : 0)) * 16;
-    ld_koff[i] = (uint32_t)r * (uint32_t)p.k_s + (uint32_t)ld_kchunk[i];
-    ld_voff[i] = (uint32_t)r * (uint32_t)p.v_s + (uint32_t)ld_vchunk[i];
+    int r; uint32_t kc, vc;
+    ld_place(i, r, kc, vc);
+    ld_koff[i] = (uint32_t)r * ks32 + kc;
+    ld_voff[i] = (uint32_t)r * vs32 + vc;
   }
   const uint32_t lds_k_addr = (uint32_t)(uintptr_t)HBSA_AS3(lds_k);
-  const uint32_t lds_v_addr = (uint32_t)(uintptr_t)HBSA_AS3(lds_v);
   // kbase / vbase: wavefront-uniform address of the tile's first key row (for this kv head).
   // 16 bytes per lane go straight from global memory into LDS at (M0 + 16 * lane); the global
-  // address is a scalar base plus a 32-bit per-lane offset.
-  auto dma16 = [&](const char *sbase, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+  // address is a scalar base plus a 32-bit per-lane offset.  The V buffers follow the K buffers.
+  auto dma16 = [&](auto off_, const char *sbase, uint32_t voff, uint32_t lds_addr) {
+    constexpr int off = decltype(off_)::value;
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
-                 : "s"(lds_addr), "v"(voff), "s"(sbase)
-                 : "memory", "m0");
+                 : "s"(lds_addr), "v"(voff), "s"(sbase), "n"(off)
+                 : "memory", "m0", "scc");
+  };
+  auto tile_ptr = [&](const char *base, int tok, uint32_t stride) {   // tok >= 0
+    return base + (uint64_t)(uint32_t)tok * (uint64_t)stride;
   };
   auto issue_loads = [&](int buf, const char *kbase, const char *vbase, int valid) {
-#pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-      uint32_t ko = ld_koff[i], vo = ld_voff[i];
-      if (valid != kTileKeys) {   // ragged tail of a run: rows past the end re-read the last valid row (masked later)
-        const uint32_t r = (uint32_t)min(ld_row[i], valid - 1);
-        ko = r * (uint32_t)p.k_s + (uint32_t)ld_kchunk[i];
-        vo = r * (uint32_t)p.v_s + (uint32_t)ld_vchunk[i];
-      }
-      const uint32_t lds_off = (uint32_t)(buf * TILE_BYTES + (i * 4 + wave) * 1024);
-      dma16(kbase, ko, lds_k_addr + lds_off);
-      dma16(vbase, vo, lds_v_addr + lds_off);
+    const uint32_t l0 = lds_k_addr + (uint32_t)(buf * TILE_BYTES) + (uint32_t)wave * 1024u;
+    if (valid == kTileKeys) {
+      static_for<0, LOADS>([&](auto i_) {
+        constexpr int i = decltype(i_)::value;
+        dma16(std::integral_constant<int, i * 4096>{}, kbase, ld_koff[i], l0);
+        dma16(std::integral_constant<int, 2 * TILE_BYTES + i * 4096>{}, vbase, ld_voff[i], l0);
+      });
+    } else {   // ragged tail of a run: rows past the end re-read the last valid row (masked later)
+      static_for<0, LOADS>([&](auto i_) {
+        constexpr int i = decltype(i_)::value;
+        int r; uint32_t kc, vc;
+        ld_place(i, r, kc, vc);
+        r = min(r, valid - 1);
+        dma16(std::integral_constant<int, i * 4096>{}, kbase, (uint32_t)r * ks32 + kc, l0);
+        dma16(std::integral_constant<int, 2 * TILE_BYTES + i * 4096>{}, vbase, (uint32_t)r * vs32 + vc, l0);
+      });
     }
   };
 
@@ -515,6 +525,31 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   const int v_lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
   const int v_swz = (CPR >= 8) ? (((v_key / RPG) % (CPR / 4)) << 2) : 0;
   const int v_rd = v_key * RB + ((v_lc | v_swz) << 4) + 8 * (lane & 1);
+
+  // Absolute LDS addresses of this lane's operand reads in the CURRENT tile buffer: one per k-step
+  // for K, one per 32-dim block for V.  flip_buffers() moves them to the other buffer with one add
+  // each (the two buffers of K, and of V, are TILE_BYTES apart), so the per-tile path has no
+  // address arithmetic besides that.
+  uint32_t k_addr[KSTEPS], v_addr[DT];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) k_addr[ks] = lds_k_addr + (uint32_t)(k_rd ^ (ks * 32));
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) v_addr[dt] = lds_k_addr + 2 * TILE_BYTES + (uint32_t)(v_rd ^ (dt * 64));
+  int buf = 0;
+  auto flip_buffers = [&]() {
+    buf ^= 1;
+    const uint32_t step = buf ? (uint32_t)TILE_BYTES : (uint32_t)-TILE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      k_addr[ks] += step;
+      asm volatile("" : "+v"(k_addr[ks]));   // keep it in its register instead of recomputing it per read
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      v_addr[dt] += step;
+      asm volatile("" : "+v"(v_addr[dt]));
+    }
+  };
 
   auto hdr_word = [&](int c, int i) { return __builtin_amdgcn_readfirstlane(lds_hdr[c * H_WORDS + i]); };
   // this wave's slice of an item: q head, first row inside the q block, rows
@@ -532,14 +567,13 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   // ------------------------------------------------------------------ first item
   int c = 0;   // list / header of the current item
   if (hdr_word(0, H_HK) < 0) return;
-  int buf = 0;
   {
     const int total0 = hdr_word(0, H_TOTAL);
     if (total0 > 0) {
       const int e = __builtin_amdgcn_readfirstlane(lds_list[0]);
-      const int64_t tok = hdr_word(0, H_KEY_BEGIN) + ((e >> 6) << 4);
+      const int tok = hdr_word(0, H_KEY_BEGIN) + ((e >> 6) << 4);
       const int hk = hdr_word(0, H_HK);
-      issue_loads(0, p.k + (int64_t)hk * p.k_h + tok * p.k_s, p.v + (int64_t)hk * p.v_h + tok * p.v_s, (e & 63) + 1);
+      issue_loads(0, tile_ptr(p.k + (int64_t)hk * p.k_h, tok, ks32), tile_ptr(p.v + (int64_t)hk * p.v_h, tok, vs32), (e & 63) + 1);
     }
   }
   short8v qf[KSTEPS];   // Q^T fragments (B operand): lane holds query l32, d = 16*ks + 8*g32 .. +7
@@ -615,15 +649,15 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
           } else {
             e1 = __builtin_amdgcn_readlane(held, (t + 1) & 63);
           }
-          const int64_t tok = (e1 >> 6) << 4;
-          issue_loads(buf ^ 1, kg + tok * p.k_s, vg + tok * p.v_s, (e1 & 63) + 1);
+          const int tok = (e1 >> 6) << 4;
+          issue_loads(buf ^ 1, tile_ptr(kg, tok, ks32), tile_ptr(vg, tok, vs32), (e1 & 63) + 1);
         } else if (last) {
           nxt_hk = hdr_word(c ^ 1, H_HK);
           if (nxt_hk >= 0 && hdr_word(c ^ 1, H_TOTAL) > 0) {
             const int e1 = __builtin_amdgcn_readfirstlane(lds_list[(c ^ 1) * kListCap]);
-            const int64_t tok = hdr_word(c ^ 1, H_KEY_BEGIN) + ((e1 >> 6) << 4);
-            issue_loads(buf ^ 1, p.k + (int64_t)nxt_hk * p.k_h + tok * p.k_s, p.v + (int64_t)nxt_hk * p.v_h + tok * p.v_s,
-                        (e1 & 63) + 1);
+            const int tok = hdr_word(c ^ 1, H_KEY_BEGIN) + ((e1 >> 6) << 4);
+            issue_loads(buf ^ 1, tile_ptr(p.k + (int64_t)nxt_hk * p.k_h, tok, ks32),
+                        tile_ptr(p.v + (int64_t)nxt_hk * p.v_h, tok, vs32), (e1 & 63) + 1);
           }
         }
 
@@ -632,8 +666,6 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
           // The tile is processed as two halves of 32 keys so that, inside one wavefront, the
           // matrix cores always have work queued while the vector ALU does the softmax of the
           // other half:   S0, max(S0) | S1 + exp(S0) | PV0 + max(S1), exp(S1) | PV1.
-          const uint32_t kt_base = (uint32_t)(uintptr_t)HBSA_AS3(lds_k + buf * TILE_BYTES);
-          const uint32_t vt_base = (uint32_t)(uintptr_t)HBSA_AS3(lds_v + buf * TILE_BYTES);
           const bool edge = valid < kTileKeys || (p.causal && kpos + valid - 1 > wave_kvis_min);
           int lim = valid;                      // keys (of this lane's query) below lim are visible
           if (p.causal) lim = min(lim, lane_kvis - kpos + 1);
@@ -651,9 +683,8 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
           auto read_k = [&](auto i_) {
             constexpr int i = decltype(i_)::value;
             constexpr int ks = i % KSTEPS;
-            const uint32_t a = kt_base + (uint32_t)(k_rd ^ (ks * 32));
-            if constexpr (i < KSTEPS) kb[i % PF] = lds_read_b128<0>(a);
-            else kb[i % PF] = lds_read_b128<32 * RB>(a);
+            if constexpr (i < KSTEPS) kb[i % PF] = lds_read_b128<0>(k_addr[ks]);
+            else kb[i % PF] = lds_read_b128<32 * RB>(k_addr[ks]);
           };
           static_for<0, PF>(read_k);
           // ---- S0 = K[0:32] . Q^T
@@ -712,9 +743,8 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
             constexpr int g = decltype(g_)::value;
             static_for<0, DT>([&](auto dt_) {
               constexpr int dt = decltype(dt_)::value;
-              const uint32_t a = vt_base + (uint32_t)(v_rd ^ (dt * 64));
-              dst[2 * dt] = lds_read_tr16_b64<g * 16 * RB>(a);
-              dst[2 * dt + 1] = lds_read_tr16_b64<g * 16 * RB + 8 * RB>(a);
+              dst[2 * dt] = lds_read_tr16_b64<g * 16 * RB>(v_addr[dt]);
+              dst[2 * dt + 1] = lds_read_tr16_b64<g * 16 * RB + 8 * RB>(v_addr[dt]);
             });
           };
           auto wait_vgroup = [&](auto n_, short4v *v) {
@@ -815,7 +845,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
             qf[ks] = __builtin_bit_cast(short8v, raw);
           }
         }
-        buf ^= 1;
+        flip_buffers();
       }
       chunk_base += n;
       if (chunk_base >= total) break;
@@ -833,8 +863,8 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
       __syncthreads();
       {   // nothing is in flight here: fetch the chunk's first tile
         const int e = __builtin_amdgcn_readfirstlane(lds_list[c * kListCap]);
-        const int64_t tok = (e >> 6) << 4;
-        issue_loads(buf, kg + tok * p.k_s, vg + tok * p.v_s, (e & 63) + 1);
+        const int tok = (e >> 6) << 4;
+        issue_loads(buf, tile_ptr(kg, tok, ks32), tile_ptr(vg, tok, vs32), (e & 63) + 1);
       }
     }
 
@@ -866,8 +896,8 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
       if (nxt_hk >= 0) {
         if (hdr_word(c ^ 1, H_TOTAL) > 0) {
           const int e1 = __builtin_amdgcn_readfirstlane(lds_list[(c ^ 1) * kListCap]);
-          const int64_t tok = hdr_word(c ^ 1, H_KEY_BEGIN) + ((e1 >> 6) << 4);
-          issue_loads(buf, p.k + (int64_t)nxt_hk * p.k_h + tok * p.k_s, p.v + (int64_t)nxt_hk * p.v_h + tok * p.v_s,
+          const int tok = hdr_word(c ^ 1, H_KEY_BEGIN) + ((e1 >> 6) << 4);
+          issue_loads(buf, tile_ptr(p.k + (int64_t)nxt_hk * p.k_h, tok, ks32), tile_ptr(p.v + (int64_t)nxt_hk * p.v_h, tok, vs32),
                       (e1 & 63) + 1);
         }
         bool act; int hq1, r01, nr1;
@@ -1006,6 +1036,10 @@ int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out, void *w
     if (strides[i] % 8 != 0)
       return fail(HBSA_ERR_INVALID_ARGUMENT, "stride %d (%lld elements) is not a multiple of 8 (16-byte rows)", i,
                   (long long)strides[i]);
+  // the tile loads address a 64-row tile with 32-bit byte offsets from its first row
+  if (strides[2] < 0 || strides[4] < 0 || strides[2] > (1 << 24) || strides[4] > (1 << 24))
+    return fail(HBSA_ERR_UNSUPPORTED, "k/v token stride (%lld, %lld elements) outside [0, 2^24]", (long long)strides[2],
+                (long long)strides[4]);
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
     return fail(HBSA_ERR_INVALID_ARGUMENT, "q/k/v/out must be 16-byte aligned");
   if ((uintptr_t)workspace & 255) return fail(HBSA_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
@@ -1067,6 +1101,10 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32
     if (strides[i] % 8 != 0)
       return fail(HBSA_ERR_INVALID_ARGUMENT, "stride %d (%lld elements) is not a multiple of 8 (16-byte rows)", i,
                   (long long)strides[i]);
+  // the tile loads address a 64-row tile with 32-bit byte offsets from its first row
+  if (strides[2] < 0 || strides[4] < 0 || strides[2] > (1 << 24) || strides[4] > (1 << 24))
+    return fail(HBSA_ERR_UNSUPPORTED, "k/v token stride (%lld, %lld elements) outside [0, 2^24]", (long long)strides[2],
+                (long long)strides[4]);
   int rc = hbsa_fwd_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_to_batch, cu_num_q_block, cu_num_k_block,
                             workspace, workspace_bytes, batch, nhead_k, num_q_block, num_k_block, q_block_size,
                             k_block_size, causal, strides + 8, stream);
