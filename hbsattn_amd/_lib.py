@@ -6,10 +6,11 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhbsattn_amd.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 DTYPE_BF16 = 0
 DTYPE_F16 = 1
+DTYPE_F32 = 2
 
 _lib = None
 
@@ -36,6 +37,8 @@ def load() -> ctypes.CDLL:
     lib.hbsa_last_error.argtypes = []
     lib.hbsa_fwd_workspace_bytes.restype = ctypes.c_size_t
     lib.hbsa_fwd_workspace_bytes.argtypes = [ctypes.c_int32] * 3
+    lib.hbsa_fwd_workspace_bytes_dtype.restype = ctypes.c_size_t
+    lib.hbsa_fwd_workspace_bytes_dtype.argtypes = [ctypes.c_int32] * 8
     vp = ctypes.c_void_p
     lib.hbsa_fwd.restype = ctypes.c_int
     lib.hbsa_fwd.argtypes = ([vp] * 11 + [ctypes.c_size_t] + [ctypes.c_int32] * 12 + [ctypes.c_float]

@@ -44,6 +44,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
@@ -89,8 +90,8 @@ struct FwdParams {
   int32_t wps;    // wave slots per q head = ceil(q_block_size / 32)
   int32_t nsub;   // workgroups per (kv head, q block) = ceil(ratio * wps / 4)
   uint32_t q_sign;  // 0x80008000 when softmax_scale < 0 (Q is negated, |scale| used)
-  float c;        // |softmax_scale| * log2(e)
-  float lag;      // kLazyRescaleLog2 / c, in raw score units
+  float c;        // |softmax_scale| * log2(e); the kernel reads the launch's value from sched
+  int32_t f32;    // fp32 inputs staged as fp16: the setup kernel derives the constants from the maxima
   int32_t nhead_k;
   struct Sched *sched;
 };
@@ -213,11 +214,84 @@ __device__ __forceinline__ float half_sum(float x) {
 // --------------------------------------------------------------------------------------
 struct Sched {
   uint32_t qnext[8];   // next unclaimed entry of each queue
-  uint32_t pad[56];
+  // softmax constants the attention kernel reads at its start (written by hbsa_setup_kernel)
+  float c;             // |softmax_scale| * log2(e), divided by the q and k staging multipliers for fp32 inputs
+  float lag;           // kLazyRescaleLog2 / c, in raw score units
+  float out_mul;       // fp32 inputs: 1 / (v staging multiplier); 1 otherwise
+  // fp32 inputs only: bit patterns of max|x| over q, k, v and the power-of-two staging multipliers
+  uint32_t amax[3];
+  float in_mul[3];
+  uint32_t pad[47];
 };
+static_assert(sizeof(Sched) == 256, "Sched is one 256-byte slot of the workspace");
 
-__global__ void hbsa_reset_kernel(Sched *s) {
+// Queue counters and softmax constants for one attention launch (a kernel, not a memset, so that
+// the launches of a call can be captured in a graph).  For fp32 inputs the constants follow from
+// the maxima the absmax kernels left in s->amax.
+__global__ void hbsa_setup_kernel(Sched *s, float c, int f32) {
   if (threadIdx.x < 8) s->qnext[threadIdx.x] = 0;
+  if (threadIdx.x != 0) return;
+  float out_mul = 1.f;
+  if (f32) {
+    // Each tensor is staged as fp16 after multiplication by a power of two that brings its largest
+    // magnitude into [2^14, 2^15): exact, and as far from fp16's overflow and underflow as possible.
+    float mul[3];
+    for (int i = 0; i < 3; ++i) {
+      const int e = (int)((s->amax[i] >> 23) & 255u);   // biased exponent of max|x|
+      int sh = 14 - (e - 127);
+      if (e == 0 || e == 255) sh = 0;                   // all zero (or denormal), inf or nan: leave as is
+      sh = sh > 126 ? 126 : (sh < -126 ? -126 : sh);    // 2^sh and its reciprocal stay normal numbers
+      mul[i] = __builtin_ldexpf(1.f, sh);
+      s->in_mul[i] = mul[i];
+    }
+    c = c / mul[0] / mul[1];
+    if (!(c >= 1.2e-38f)) c = 1.2e-38f;                 // keep -inf * c == -inf
+    if (c > 3e38f) c = 3e38f;
+    out_mul = 1.f / mul[2];
+  }
+  s->c = c;
+  s->lag = kLazyRescaleLog2 / c;
+  s->out_mul = out_mul;
+}
+
+__global__ void hbsa_f32_begin_kernel(Sched *s) {
+  if (threadIdx.x < 3) s->amax[threadIdx.x] = 0;
+}
+
+// fp32 staging.  A tensor is [tokens, heads, D] with element strides (tok_s, head_s), rows of D
+// contiguous floats, 16-byte aligned; one thread handles 4 consecutive floats.
+struct F32Tensor {
+  const float *x;
+  int64_t tok_s, head_s;
+  int32_t heads, dshift;   // dshift = log2(D / 4)
+  int64_t quads;           // tokens * heads * D / 4
+};
+__device__ __forceinline__ const float *f32_quad_ptr(const F32Tensor &t, int64_t i) {
+  const int64_t row = i >> t.dshift;
+  const int dq = (int)(i & ((1 << t.dshift) - 1));
+  return t.x + (row / t.heads) * t.tok_s + (row % t.heads) * t.head_s + dq * 4;
+}
+// max |x| as a bit pattern (for non-negative floats the integer order is the float order)
+__global__ __launch_bounds__(256) void hbsa_f32_absmax_kernel(F32Tensor t, uint32_t *amax) {
+  uint32_t m = 0;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < t.quads; i += (int64_t)gridDim.x * 256) {
+    const u32x4 v = *(const u32x4 *)f32_quad_ptr(t, i);
+    m = max(max(m, v.x & 0x7fffffffu), max(max(v.y & 0x7fffffffu, v.z & 0x7fffffffu), v.w & 0x7fffffffu));
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off));
+  if ((threadIdx.x & 63) == 0 && m != 0) atomicMax(amax, m);
+}
+// fp16 copy, contiguous [tokens, heads, D], of x * *mul
+__global__ __launch_bounds__(256) void hbsa_f32_stage_kernel(F32Tensor t, const float *mul, uint32_t *dst) {
+  const float m = *mul;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < t.quads; i += (int64_t)gridDim.x * 256) {
+    const float *src = f32_quad_ptr(t, i);
+    u32x2 w;
+    w.x = ElemF16::pack2(src[0] * m, src[1] * m);
+    w.y = ElemF16::pack2(src[2] * m, src[3] * m);
+    *(u32x2 *)(dst + 2 * i) = w;
+  }
 }
 
 #ifndef HBSA_INTERLEAVE_C
@@ -368,8 +442,9 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-template <int D, typename E>
+template <int D, typename E, bool OUT32>
 __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
+  // OUT32: fp32 output (the fp32-input path; q/k/v are then fp16 staging copies)
   constexpr int RB = D * 2;            // row bytes
   constexpr int CPR = RB / 16;         // 16-byte chunks per row
   constexpr int RPG = 16 / CPR > 0 ? 16 / CPR : 1;  // rows per 256-byte bank sweep
@@ -387,6 +462,12 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g32 = lane >> 5;   // which half of the wavefront
   const int l32 = lane & 31;   // query within the wave slot / key row within a sub-tile
+
+  // softmax constants of this launch (uniform; written by the setup kernel that precedes it)
+  const float sm_c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, p.sched->c)));
+  const float sm_lag = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, p.sched->lag)));
+  const float sm_out_mul =
+      __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, p.sched->out_mul)));
 
   // ------------------------------------------------------------------ scheduler (wavefront 0)
   const int nq = p.nhead_k < 8 ? p.nhead_k : 8;                       // queues that hold work
@@ -711,10 +792,10 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 #pragma unroll
             for (int i = 2; i < 16; i += 2) mx = max3(mx, sh[i], sh[i + 1]);
             mx = half_max(mx);
-            const bool grow = mx > m_run + p.lag;
+            const bool grow = mx > m_run + sm_lag;
             if (__builtin_amdgcn_ballot_w64(grow) != 0) {
               const float m_new = grow ? mx : m_run;
-              const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * p.c) : 1.f;
+              const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * sm_c) : 1.f;
               l_run *= alpha;
 #pragma unroll
               for (int dt = 0; dt < DT; ++dt)
@@ -725,14 +806,14 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
           };
           // exponentials of one half, packed to the element type (two groups of 16 keys), row sum
           auto half_exp = [&](const f32x16 &sh, short8v &p_lo, short8v &p_hi) {
-            const float mc = (m_run == -INFINITY) ? 0.f : m_run * p.c;
+            const float mc = (m_run == -INFINITY) ? 0.f : m_run * sm_c;
             u32x4 w[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
               for (int q4 = 0; q4 < 4; ++q4) {
-                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sh[8 * j + 2 * q4], p.c, -mc));
-                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sh[8 * j + 2 * q4 + 1], p.c, -mc));
+                const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sh[8 * j + 2 * q4], sm_c, -mc));
+                const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sh[8 * j + 2 * q4 + 1], sm_c, -mc));
                 w[j][q4] = E::pack2(e0, e1);
                 // fp32 adds, not v_dot2c: the dot instructions share the matrix pipeline and would
                 // stall the MFMAs of the wavefront's neighbour on the SIMD
@@ -796,10 +877,10 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 #pragma unroll
             for (int i = 2; i < 16; i += 2) mx = max3(mx, s1[i], s1[i + 1]);
             mx = half_max(mx);
-            const bool grow = mx > m_run + p.lag;
+            const bool grow = mx > m_run + sm_lag;
             if (__builtin_amdgcn_ballot_w64(grow) != 0) {
               const float m_new = grow ? mx : m_run;
-              const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * p.c) : 1.f;
+              const float alpha = grow ? __builtin_amdgcn_exp2f((m_run - m_new) * sm_c) : 1.f;
               l_run *= alpha;
 #pragma unroll
               for (int dt = 0; dt < DT; ++dt)
@@ -876,15 +957,26 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
       const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
       if (l32 < nrows) {
         char *orow = p.out + (int64_t)(row_begin + row0 + l32) * p.o_s + (int64_t)hq * p.o_h;
+        if constexpr (OUT32) {
+          const float f = inv * sm_out_mul;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+          for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int i4 = 0; i4 < 4; ++i4) {
-            u32x2 w;
-            w.x = E::pack2(o[dt][4 * i4 + 0] * inv, o[dt][4 * i4 + 1] * inv);
-            w.y = E::pack2(o[dt][4 * i4 + 2] * inv, o[dt][4 * i4 + 3] * inv);
-            *(u32x2 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 2) = w;
-          }
+            for (int i4 = 0; i4 < 4; ++i4) {
+              f32x4 w = {o[dt][4 * i4 + 0] * f, o[dt][4 * i4 + 1] * f, o[dt][4 * i4 + 2] * f, o[dt][4 * i4 + 3] * f};
+              *(f32x4 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 4) = w;
+            }
+        } else {
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+              u32x2 w;
+              w.x = E::pack2(o[dt][4 * i4 + 0] * inv, o[dt][4 * i4 + 1] * inv);
+              w.y = E::pack2(o[dt][4 * i4 + 2] * inv, o[dt][4 * i4 + 3] * inv);
+              *(u32x2 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 2) = w;
+            }
+        }
       }
     }
 
@@ -936,6 +1028,33 @@ inline int words_per_row(int num_k_block) { return 2 * ((num_k_block + 63) / 64)
 inline size_t sched_offset(int num_q_block) { return align_up((size_t)num_q_block * sizeof(QBlockInfo), 256); }
 inline size_t bits_offset(int num_q_block) { return sched_offset(num_q_block) + align_up(sizeof(Sched), 256); }
 
+// rows must be 16-byte aligned: strides (in elements) multiples of 8 for 16-bit types, of 4 for fp32
+int check_strides(const int64_t *strides, bool f32) {
+  const int unit = f32 ? 4 : 8;
+  for (int i = 0; i < 8; ++i)
+    if (strides[i] % unit != 0)
+      return fail(HBSA_ERR_INVALID_ARGUMENT, "stride %d (%lld elements) is not a multiple of %d (16-byte rows)", i,
+                  (long long)strides[i], unit);
+  // 16-bit inputs: the tile loads address a 64-row tile with 32-bit byte offsets from its first row
+  if (strides[2] < 0 || strides[4] < 0 || strides[2] > (1 << 24) || strides[4] > (1 << 24))
+    return fail(HBSA_ERR_UNSUPPORTED, "k/v token stride (%lld, %lld elements) outside [0, 2^24]", (long long)strides[2],
+                (long long)strides[4]);
+  return 0;
+}
+
+// fp32 inputs: bytes of one fp16 staging copy [tokens, heads, D], placed after the bit words
+inline size_t f32_stage_bytes(int64_t tokens, int64_t heads, int64_t d) { return align_up((size_t)(tokens * heads * d * 2), 256); }
+
+// tensor i (0 q, 1 k, 2 v) of an fp32 call
+F32Tensor f32_tensor(int i, const void *q, const void *k, const void *v, const int64_t *strides, int total_q, int total_k,
+                     int nhead_q, int nhead_k, int headdim) {
+  const int dshift = headdim == 32 ? 3 : headdim == 64 ? 4 : 5;
+  const void *x = i == 0 ? q : i == 1 ? k : v;
+  const int64_t tokens = i == 0 ? total_q : total_k;
+  const int heads = i == 0 ? nhead_q : nhead_k;
+  return {(const float *)x, strides[2 * i], strides[2 * i + 1], heads, dshift, tokens * heads * headdim / 4};
+}
+
 int persistent_grid(const void *kernel, int lds_bytes) {
   int dev = 0, cus = 0, per_cu = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
@@ -946,10 +1065,10 @@ int persistent_grid(const void *kernel, int lds_bytes) {
   return cus * per_cu;
 }
 
-template <int D, typename E>
+template <int D, typename E, bool OUT32>
 int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
   constexpr int lds_bytes = 4 * kTileKeys * D * 2 + 2 * H_WORDS * 4 + 2 * kListCap * 4;
-  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E>);
+  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E, OUT32>);
   static thread_local int resident = 0;   // workgroups that fit the device at once
   if (resident == 0) {
     hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -958,8 +1077,8 @@ int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
     if (resident <= 0) return fail(HBSA_ERR_UNSUPPORTED, "could not size the persistent grid");
   }
   const int grid = (int)(items < resident ? items : resident);
-  hipLaunchKernelGGL(hbsa_reset_kernel, dim3(1), dim3(64), 0, stream, fp.sched);
-  hipLaunchKernelGGL((hbsa_fwd_kernel<D, E>), dim3(grid), dim3(kThreads), lds_bytes, stream, fp);
+  hipLaunchKernelGGL(hbsa_setup_kernel, dim3(1), dim3(64), 0, stream, fp.sched, fp.c, fp.f32);
+  hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32>), dim3(grid), dim3(kThreads), lds_bytes, stream, fp);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail((int)e, "hbsa_fwd_kernel launch: %s", hipGetErrorString(e));
   return 0;
@@ -977,6 +1096,14 @@ size_t hbsa_fwd_workspace_bytes(int32_t nhead_k, int32_t num_q_block, int32_t nu
   if (nhead_k <= 0 || num_q_block <= 0 || num_k_block <= 0) return 256;
   const size_t bits = align_up((size_t)nhead_k * num_q_block * words_per_row(num_k_block) * sizeof(uint32_t), 256);
   return bits_offset(num_q_block) + bits;
+}
+
+size_t hbsa_fwd_workspace_bytes_dtype(int32_t dtype, int32_t total_q, int32_t total_k, int32_t nhead_q,
+                                      int32_t nhead_k, int32_t headdim, int32_t num_q_block, int32_t num_k_block) {
+  size_t n = hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block);
+  if (dtype == HBSA_DTYPE_F32 && total_q > 0 && total_k > 0 && nhead_q > 0 && nhead_k > 0 && headdim > 0)
+    n += f32_stage_bytes(total_q, nhead_q, headdim) + 2 * f32_stage_bytes(total_k, nhead_k, headdim);
+  return n;
 }
 
 int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens, const uint8_t *block_mask,
@@ -1030,33 +1157,49 @@ int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out, void *w
                 q_block_size, k_block_size);
   if (headdim != 32 && headdim != 64 && headdim != 128)
     return fail(HBSA_ERR_UNSUPPORTED, "headdim %d not in {32, 64, 128}", headdim);
-  if (dtype != HBSA_DTYPE_BF16 && dtype != HBSA_DTYPE_F16)
+  if (dtype != HBSA_DTYPE_BF16 && dtype != HBSA_DTYPE_F16 && dtype != HBSA_DTYPE_F32)
     return fail(HBSA_ERR_UNSUPPORTED, "dtype code %d not supported", dtype);
   if (num_k_block <= 0 || total_k <= 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "no keys");
   if (!std::isfinite(softmax_scale)) return fail(HBSA_ERR_INVALID_ARGUMENT, "softmax_scale is not finite");
-  for (int i = 0; i < 8; ++i)
-    if (strides[i] % 8 != 0)
-      return fail(HBSA_ERR_INVALID_ARGUMENT, "stride %d (%lld elements) is not a multiple of 8 (16-byte rows)", i,
-                  (long long)strides[i]);
-  // the tile loads address a 64-row tile with 32-bit byte offsets from its first row
-  if (strides[2] < 0 || strides[4] < 0 || strides[2] > (1 << 24) || strides[4] > (1 << 24))
-    return fail(HBSA_ERR_UNSUPPORTED, "k/v token stride (%lld, %lld elements) outside [0, 2^24]", (long long)strides[2],
-                (long long)strides[4]);
+  const bool f32 = dtype == HBSA_DTYPE_F32;
+  if (int rc = check_strides(strides, f32)) return rc;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
     return fail(HBSA_ERR_INVALID_ARGUMENT, "q/k/v/out must be 16-byte aligned");
   if ((uintptr_t)workspace & 255) return fail(HBSA_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
-  const size_t need = hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block);
+  const size_t base = hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block);
+  const size_t need = hbsa_fwd_workspace_bytes_dtype(dtype, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
+                                                     num_k_block);
   if (workspace_bytes < need)
     return fail(HBSA_ERR_WORKSPACE_TOO_SMALL, "workspace %zu bytes < required %zu", workspace_bytes, need);
 
+  hipStream_t st = (hipStream_t)stream;
   FwdParams fp;
   fp.q = (const char *)q; fp.k = (const char *)k; fp.v = (const char *)v; fp.out = (char *)out;
   fp.info = (const QBlockInfo *)workspace;
   fp.bits = (const uint32_t *)((const char *)workspace + bits_offset(num_q_block));
   fp.sched = (Sched *)((char *)workspace + sched_offset(num_q_block));
   fp.nhead_k = nhead_k;
-  fp.q_s = strides[0] * 2; fp.q_h = strides[1] * 2; fp.k_s = strides[2] * 2; fp.k_h = strides[3] * 2;
-  fp.v_s = strides[4] * 2; fp.v_h = strides[5] * 2; fp.o_s = strides[6] * 2; fp.o_h = strides[7] * 2;
+  fp.f32 = f32 ? 1 : 0;
+  if (f32) {
+    // fp16 staging copies (contiguous) behind the bit words; the attention kernel reads those
+    char *sq = (char *)workspace + base;
+    char *sk = sq + f32_stage_bytes(total_q, nhead_q, headdim);
+    char *sv = sk + f32_stage_bytes(total_k, nhead_k, headdim);
+    hipLaunchKernelGGL(hbsa_f32_begin_kernel, dim3(1), dim3(64), 0, st, fp.sched);
+    for (int i = 0; i < 3; ++i) {
+      const F32Tensor t = f32_tensor(i, q, k, v, strides, total_q, total_k, nhead_q, nhead_k, headdim);
+      const unsigned nb = (unsigned)std::min<int64_t>((t.quads + 255) / 256, 4096);
+      hipLaunchKernelGGL(hbsa_f32_absmax_kernel, dim3(nb), dim3(256), 0, st, t, &fp.sched->amax[i]);
+    }
+    fp.q = sq; fp.k = sk; fp.v = sv;
+    fp.q_s = (int64_t)nhead_q * headdim * 2; fp.q_h = headdim * 2;
+    fp.k_s = (int64_t)nhead_k * headdim * 2; fp.k_h = headdim * 2;
+    fp.v_s = fp.k_s; fp.v_h = fp.k_h;
+    fp.o_s = strides[6] * 4; fp.o_h = strides[7] * 4;
+  } else {
+    fp.q_s = strides[0] * 2; fp.q_h = strides[1] * 2; fp.k_s = strides[2] * 2; fp.k_h = strides[3] * 2;
+    fp.v_s = strides[4] * 2; fp.v_h = strides[5] * 2; fp.o_s = strides[6] * 2; fp.o_h = strides[7] * 2;
+  }
   fp.nqb = num_q_block; fp.ratio = nhead_q / nhead_k; fp.kbs = k_block_size; fp.wpr = words_per_row(num_k_block);
   fp.causal = causal ? 1 : 0;
   fp.wps = (q_block_size + kWaveRows - 1) / kWaveRows;
@@ -1065,16 +1208,30 @@ int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out, void *w
   float c = std::fabs(softmax_scale) * kLog2e;
   if (c < 1e-30f) c = 1e-30f;  // scale 0: uniform weights over the visible keys, and -inf * c stays -inf
   fp.c = c;
-  fp.lag = kLazyRescaleLog2 / c;
   const long long items = (long long)nhead_k * num_q_block * fp.nsub;
   if (items > 0x7fffffffLL) return fail(HBSA_ERR_UNSUPPORTED, "too many work items (%lld)", items);
 
-  hipStream_t st = (hipStream_t)stream;
+  if (f32) {
+    // setup (multipliers from the maxima), staging, attention: the launch order on the stream is the
+    // dependency order
+    hipLaunchKernelGGL(hbsa_setup_kernel, dim3(1), dim3(64), 0, st, fp.sched, fp.c, 1);
+    const char *dst[3] = {fp.q, fp.k, fp.v};
+    for (int i = 0; i < 3; ++i) {
+      const F32Tensor t = f32_tensor(i, q, k, v, strides, total_q, total_k, nhead_q, nhead_k, headdim);
+      const unsigned nb = (unsigned)std::min<int64_t>((t.quads + 255) / 256, 8192);
+      hipLaunchKernelGGL(hbsa_f32_stage_kernel, dim3(nb), dim3(256), 0, st, t, &fp.sched->in_mul[i], (uint32_t *)dst[i]);
+    }
+    switch (headdim) {
+      case 32: return launch_fwd<32, ElemF16, true>(fp, items, st);
+      case 64: return launch_fwd<64, ElemF16, true>(fp, items, st);
+      default: return launch_fwd<128, ElemF16, true>(fp, items, st);
+    }
+  }
   const bool bf = dtype == HBSA_DTYPE_BF16;
   switch (headdim) {
-    case 32: return bf ? launch_fwd<32, ElemBF16>(fp, items, st) : launch_fwd<32, ElemF16>(fp, items, st);
-    case 64: return bf ? launch_fwd<64, ElemBF16>(fp, items, st) : launch_fwd<64, ElemF16>(fp, items, st);
-    default: return bf ? launch_fwd<128, ElemBF16>(fp, items, st) : launch_fwd<128, ElemF16>(fp, items, st);
+    case 32: return bf ? launch_fwd<32, ElemBF16, false>(fp, items, st) : launch_fwd<32, ElemF16, false>(fp, items, st);
+    case 64: return bf ? launch_fwd<64, ElemBF16, false>(fp, items, st) : launch_fwd<64, ElemF16, false>(fp, items, st);
+    default: return bf ? launch_fwd<128, ElemBF16, false>(fp, items, st) : launch_fwd<128, ElemF16, false>(fp, items, st);
   }
 }
 
@@ -1094,19 +1251,18 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32
     return fail(HBSA_ERR_INVALID_ARGUMENT, "nhead_q (%d) must be divisible by nhead_k (%d)", nhead_q, nhead_k);
   if (headdim != 32 && headdim != 64 && headdim != 128)
     return fail(HBSA_ERR_UNSUPPORTED, "headdim %d not in {32, 64, 128}", headdim);
-  if (dtype != HBSA_DTYPE_BF16 && dtype != HBSA_DTYPE_F16)
+  if (dtype != HBSA_DTYPE_BF16 && dtype != HBSA_DTYPE_F16 && dtype != HBSA_DTYPE_F32)
     return fail(HBSA_ERR_UNSUPPORTED, "dtype code %d not supported", dtype);
   if (!std::isfinite(softmax_scale)) return fail(HBSA_ERR_INVALID_ARGUMENT, "softmax_scale is not finite");
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
     return fail(HBSA_ERR_INVALID_ARGUMENT, "q/k/v/out must be 16-byte aligned");
-  for (int i = 0; i < 8; ++i)
-    if (strides[i] % 8 != 0)
-      return fail(HBSA_ERR_INVALID_ARGUMENT, "stride %d (%lld elements) is not a multiple of 8 (16-byte rows)", i,
-                  (long long)strides[i]);
-  // the tile loads address a 64-row tile with 32-bit byte offsets from its first row
-  if (strides[2] < 0 || strides[4] < 0 || strides[2] > (1 << 24) || strides[4] > (1 << 24))
-    return fail(HBSA_ERR_UNSUPPORTED, "k/v token stride (%lld, %lld elements) outside [0, 2^24]", (long long)strides[2],
-                (long long)strides[4]);
+  if (int rc = check_strides(strides, dtype == HBSA_DTYPE_F32)) return rc;
+  {
+    const size_t need = hbsa_fwd_workspace_bytes_dtype(dtype, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
+                                                       num_k_block);
+    if (workspace_bytes < need)
+      return fail(HBSA_ERR_WORKSPACE_TOO_SMALL, "workspace %zu bytes < required %zu", workspace_bytes, need);
+  }
   int rc = hbsa_fwd_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_to_batch, cu_num_q_block, cu_num_k_block,
                             workspace, workspace_bytes, batch, nhead_k, num_q_block, num_k_block, q_block_size,
                             k_block_size, causal, strides + 8, stream);

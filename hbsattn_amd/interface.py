@@ -18,7 +18,7 @@ from . import _lib
 from .utils import calculate_blocks
 
 _NATIVE_HEADDIMS = (32, 64, 128)
-_DTYPE_CODES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16}
+_DTYPE_CODES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16, torch.float32: _lib.DTYPE_F32}
 
 
 def _as_int32(t: torch.Tensor) -> torch.Tensor:
@@ -29,7 +29,9 @@ def _as_int32(t: torch.Tensor) -> torch.Tensor:
 
 def _rows_ok(t: torch.Tensor) -> bool:
     """16-byte aligned rows with a unit head-dim stride are what the kernels load."""
-    return (t.stride(2) == 1 and t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0 and t.data_ptr() % 16 == 0)
+    unit = 16 // t.element_size()
+    return (t.stride(2) == 1 and t.stride(0) % unit == 0 and t.stride(1) % unit == 0 and t.data_ptr() % 16 == 0
+            and 0 <= t.stride(0) <= 1 << 24)
 
 
 def _pad_headdim(t: torch.Tensor, d_pad: int) -> torch.Tensor:
@@ -59,8 +61,10 @@ def _check_block_sizes(q_block_size, k_block_size):
 
 
 def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, num_q_block,
-                 q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block) -> PreparedMask:
-    """Runs the pre-pass kernel (``hbsa_fwd_prepare``) on the current stream."""
+                 q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, staging=None) -> PreparedMask:
+    """Runs the pre-pass kernel (``hbsa_fwd_prepare``) on the current stream.  ``staging`` =
+    ``(total_q, total_k, nhead_q, headdim)`` reserves the room fp32 q/k/v of that size need behind
+    the work description (``hbsa_run`` grows the workspace itself when it is missing)."""
     if not block_mask.is_cuda:
         raise RuntimeError("hbsattn_amd runs on MI355X only: block_mask must be a CUDA(HIP) tensor; there is no CPU path")
     _check_block_sizes(q_block_size, k_block_size)
@@ -68,6 +72,10 @@ def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_s
     dev = block_mask.device
     nhead_k = block_mask.shape[0]
     ws_bytes = int(lib.hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block))
+    if staging is not None:
+        total_q, total_k, nhead_q, headdim = staging
+        ws_bytes = int(lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F32, total_q, total_k, nhead_q, nhead_k, headdim,
+                                                          num_q_block, num_k_block))
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     cu_q, cu_k = _as_int32(cu_q_seqlens), _as_int32(cu_k_seqlens)
     qb2b, cu_nqb, cu_nkb = _as_int32(q_block_to_batch), _as_int32(cu_num_q_block), _as_int32(cu_num_k_block)
@@ -93,7 +101,7 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale) -> torch.Tensor:
     if not (k.dtype == q.dtype and v.dtype == q.dtype):
         raise TypeError("q, k and v must share one dtype")
     if q.dtype not in _DTYPE_CODES:
-        raise TypeError(f"hbsattn_amd: dtype {q.dtype} is not supported (bfloat16 and float16 are)")
+        raise TypeError(f"hbsattn_amd: dtype {q.dtype} is not supported (bfloat16, float16 and float32 are)")
     total_q, nhead_q, headdim = q.shape
     total_k, nhead_k = k.shape[0], k.shape[1]
     if k.shape[2] != headdim or v.shape != k.shape:
@@ -121,6 +129,13 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale) -> torch.Tensor:
     strides = (ctypes.c_int64 * 8)(q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
                                    out_run.stride(0), out_run.stride(1))
     ws = prepared.workspace
+    if q.dtype == torch.float32:   # room for the fp16 staging copies behind the work description
+        need = int(lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F32, total_q, total_k, nhead_q, nhead_k, d_run,
+                                                      prepared.num_q_block, prepared.num_k_block))
+        if ws.numel() < need:
+            grown = torch.empty(need, dtype=torch.uint8, device=ws.device)
+            grown[: ws.numel()].copy_(ws)
+            prepared.workspace = ws = grown
     with torch.cuda.device(q.device):
         rc = lib.hbsa_fwd_run(q.data_ptr(), k.data_ptr(), v.data_ptr(), out_run.data_ptr(), ws.data_ptr(), ws.numel(),
                               _DTYPE_CODES[q.dtype], total_q, total_k, nhead_q, nhead_k, d_run, prepared.num_q_block,
@@ -144,8 +159,11 @@ def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, 
     if block_mask.device != q.device:
         raise RuntimeError("q, k, v and block_mask must live on the same device")
     assert q.shape[1] % k.shape[1] == 0, "nhead_q must be divisible by nhead_k (for GQA)"
+    staging = None
+    if q.dtype == torch.float32 and q.dim() == 3 and k.dim() == 3:
+        staging = (q.shape[0], k.shape[0], q.shape[1], next((d for d in _NATIVE_HEADDIMS if d >= q.shape[2]), q.shape[2]))
     prepared = hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, num_q_block,
-                            q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block)
+                            q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, staging)
     return hbsa_run(q, k, v, prepared, softmax_scale)
 
 

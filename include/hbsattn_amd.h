@@ -16,7 +16,8 @@
  *     stream) and the calls return without synchronising;
  *   - return value 0 = success, negative = invalid argument (message available
  *     through hbsa_last_error(), which is thread-local), positive = hipError_t;
- *   - strides are in ELEMENTS; the innermost (head-dim) stride of q/k/v/out must be 1.
+ *   - strides are in ELEMENTS; the innermost (head-dim) stride of q/k/v/out must be 1 and
+ *     every row must start on a 16-byte boundary.
  */
 #ifndef HBSATTN_AMD_H_
 #define HBSATTN_AMD_H_
@@ -28,12 +29,13 @@
 extern "C" {
 #endif
 
-#define HBSA_ABI_VERSION 1
+#define HBSA_ABI_VERSION 2
 
 /* element types of q/k/v/out (reference: dtype follows the input tensors,
  * hbsattn/fwd_triton_auto_tile_size.py:272) */
 #define HBSA_DTYPE_BF16 0
 #define HBSA_DTYPE_F16 1
+#define HBSA_DTYPE_F32 2 /* see hbsa_fwd_workspace_bytes_dtype */
 
 #define HBSA_ERR_INVALID_ARGUMENT (-1)
 #define HBSA_ERR_UNSUPPORTED (-2)
@@ -55,6 +57,21 @@ const char *hbsa_last_error(void);
 size_t hbsa_fwd_workspace_bytes(int32_t nhead_k, int32_t num_q_block, int32_t num_k_block);
 
 /*
+ * The same for a given element type.  For HBSA_DTYPE_BF16 / HBSA_DTYPE_F16 it equals
+ * hbsa_fwd_workspace_bytes.  For HBSA_DTYPE_F32 (the reference accepts fp32 q/k/v, its tests use
+ * them: reference test/test_accuracy.py:24) it adds room for fp16 staging copies of q, k and v:
+ * fp32 tensors are multiplied by a power of two chosen from their largest magnitude (found on the
+ * device, no host synchronisation) and rounded to fp16, the products accumulate in fp32, the
+ * softmax runs in fp32 and `out` is written as fp32.  That is the precision class of the
+ * reference's own fp32 path (Triton's tl.dot rounds fp32 operands to tf32, which has fp16's
+ * 11-bit significand), with fp32's range kept by the scaling.
+ * hbsa_fwd_prepare needs only the hbsa_fwd_workspace_bytes prefix.
+ */
+size_t hbsa_fwd_workspace_bytes_dtype(int32_t dtype, int32_t total_q, int32_t total_k,
+                                      int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+                                      int32_t num_q_block, int32_t num_k_block);
+
+/*
  * Block-sparse attention forward.  Replaces `_forward_auto_tile_size` and
  * `_forward_fix_tile_size` + their Triton `_fwd_kernel`s (reference
  * hbsattn/fwd_triton_auto_tile_size.py:76-310, hbsattn/fwd_triton_fix_tile_size.py:30-276).
@@ -71,7 +88,7 @@ size_t hbsa_fwd_workspace_bytes(int32_t nhead_k, int32_t num_q_block, int32_t nu
  *   softmax_scale  already resolved (the caller substitutes headdim**-0.5 for None)
  *   strides     int64[11] = { q_tok, q_head, k_tok, k_head, v_tok, v_head,
  *                             out_tok, out_head, mask_head, mask_qblk, mask_kblk }
- *   workspace   >= hbsa_fwd_workspace_bytes(...) bytes, 256-byte aligned
+ *   workspace   >= hbsa_fwd_workspace_bytes_dtype(...) bytes, 256-byte aligned
  *
  * Supported: headdim in {32, 64, 128}; q_block_size, k_block_size positive multiples
  * of 16; nhead_q % nhead_k == 0; every sequence length >= 1.  Query rows with no

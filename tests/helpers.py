@@ -8,6 +8,10 @@ from oracle.dense import hbsa_oracle
 # North-star tolerance for 16-bit inputs against the fp32 masked-dense oracle.
 MAX_ABS_TOL = 2e-2
 MEAN_ABS_TOL = 2e-3
+# fp32 inputs are computed with 11-bit significands for q, k, v and p (fp32 accumulation and softmax),
+# like the reference's tf32 dot products: an order of magnitude tighter than the 16-bit bar.
+F32_MAX_ABS_TOL = 4e-3
+F32_MEAN_ABS_TOL = 3e-4
 
 
 def oracle_for(w, **kw) -> torch.Tensor:
@@ -16,11 +20,15 @@ def oracle_for(w, **kw) -> torch.Tensor:
                        w.k_block_size, w.causal, w.softmax_scale, **kw)
 
 
-def assert_close_to_oracle(out: torch.Tensor, ref: torch.Tensor, what: str = "") -> None:
+def assert_close_to_oracle(out: torch.Tensor, ref: torch.Tensor, what: str = "", max_abs: float = None,
+                           mean_abs: float = None) -> None:
+    f32 = out.dtype == torch.float32
+    max_abs = max_abs if max_abs is not None else (F32_MAX_ABS_TOL if f32 else MAX_ABS_TOL)
+    mean_abs = mean_abs if mean_abs is not None else (F32_MEAN_ABS_TOL if f32 else MEAN_ABS_TOL)
     out = out.detach().float().cpu()
     sel = ~torch.isnan(ref)
     assert sel.any(), "oracle computed nothing"
     assert torch.isfinite(out).all(), f"{what}: non-finite output"
     err = (out[sel] - ref[sel]).abs()
-    assert err.max().item() <= MAX_ABS_TOL, f"{what}: max-abs {err.max().item():.3e} > {MAX_ABS_TOL}"
-    assert err.mean().item() <= MEAN_ABS_TOL, f"{what}: mean-abs {err.mean().item():.3e} > {MEAN_ABS_TOL}"
+    assert err.max().item() <= max_abs, f"{what}: max-abs {err.max().item():.3e} > {max_abs}"
+    assert err.mean().item() <= mean_abs, f"{what}: mean-abs {err.mean().item():.3e} > {mean_abs}"

@@ -47,6 +47,17 @@ def test_workspace_bytes_is_host_only_and_monotone():
     assert c < 80 * 2 ** 20
 
 
+def test_workspace_bytes_per_dtype():
+    lib = _lib.load()
+    base = lib.hbsa_fwd_workspace_bytes(8, 64, 64)
+    args = (1000, 2000, 32, 8, 128, 64, 64)
+    assert lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_BF16, *args) == base
+    assert lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F16, *args) == base
+    f32 = lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F32, *args)
+    staged = (1000 * 32 + 2 * 2000 * 8) * 128 * 2          # fp16 copies of q, k and v
+    assert base + staged <= f32 <= base + staged + 3 * 256 and f32 % 256 == 0
+
+
 def _call_fwd(lib, **over):
     strides = (ctypes.c_int64 * 11)(4096, 128, 4096, 128, 4096, 128, 4096, 128, 1, 1, 1)
     a = dict(q=256, k=256, v=256, out=256, cu_q=256, cu_k=256, mask=256, qb2b=256, cu_nqb=256, cu_nkb=256, ws=256,

@@ -30,7 +30,7 @@ def _run(w, tile_mode="auto", with_meta=True):
 # ---------------------------------------------------------------------------------------
 # the reference's own parametrisation (reference test/test_accuracy.py:17-29), seeded
 # ---------------------------------------------------------------------------------------
-GRID = list(itertools.product([False, True], [(2, 2), (8, 2)], [None, 0.333], [torch.bfloat16, torch.float16],
+GRID = list(itertools.product([False, True], [(2, 2), (8, 2)], [None, 0.333], [torch.bfloat16, torch.float16, torch.float32],
                               [16, 32, 80], [16, 32], [True, False], [16, 18, 32]))
 
 
@@ -54,7 +54,7 @@ def test_reference_grid(tile_mode):
         assert_close_to_oracle(out, ref, what)
         assert torch.allclose(out.float().cpu(), ref.to(dtype).float(), atol=1e-2, rtol=1e-2), what
         n += 1
-    assert n >= 384
+    assert n >= 576
 
 
 # ---------------------------------------------------------------------------------------
@@ -258,7 +258,9 @@ def _call_hbsa_fwd(w, workspace_bytes=None, headdim=None):
     i32 = lambda t: t.to(torch.int32).contiguous()
     cu_q, cu_k, qb2b, cu_nqb, cu_nkb = map(i32, (w.cu_q_seqlens, w.cu_k_seqlens, qb2b, cu_nqb, cu_nkb))
     out = torch.full_like(w.q, float("nan"))
-    need = lib.hbsa_fwd_workspace_bytes(w.k.shape[1], nqb, nkb)
+    code = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}[w.q.dtype]
+    need = lib.hbsa_fwd_workspace_bytes_dtype(code, w.q.shape[0], w.k.shape[0], w.q.shape[1], w.k.shape[1], w.q.shape[2],
+                                              nqb, nkb)
     ws = torch.empty(need, dtype=torch.uint8, device=w.q.device)
     strides = (ctypes.c_int64 * 11)(w.q.stride(0), w.q.stride(1), w.k.stride(0), w.k.stride(1), w.v.stride(0),
                                     w.v.stride(1), out.stride(0), out.stride(1), *w.block_mask.stride())
@@ -266,7 +268,7 @@ def _call_hbsa_fwd(w, workspace_bytes=None, headdim=None):
     rc = lib.hbsa_fwd(w.q.data_ptr(), w.k.data_ptr(), w.v.data_ptr(), out.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),
                       w.block_mask.data_ptr(), qb2b.data_ptr(), cu_nqb.data_ptr(), cu_nkb.data_ptr(), ws.data_ptr(),
                       need if workspace_bytes is None else workspace_bytes,
-                      0 if w.q.dtype == torch.bfloat16 else 1, len(w.cu_q) - 1, w.q.shape[0], w.k.shape[0],
+                      code, len(w.cu_q) - 1, w.q.shape[0], w.k.shape[0],
                       w.q.shape[1], w.k.shape[1], w.q.shape[2] if headdim is None else headdim, nqb, nkb,
                       w.q_block_size, w.k_block_size, int(w.causal), scale, strides,
                       torch.cuda.current_stream().cuda_stream)
@@ -293,3 +295,51 @@ def test_combined_c_entry_point_rejects_bad_arguments_without_launching():
     rc, out, msg = _call_hbsa_fwd(w, headdim=48)
     assert rc == -2 and "headdim" in msg
     assert torch.isnan(out.float()).all()
+
+
+# ---------------------------------------------------------------------------------------
+# fp32 inputs (staged as scaled fp16 on the device, fp32 output)
+# ---------------------------------------------------------------------------------------
+def test_fp32_inputs_medium_problem():
+    w = make_problem(seed=31, q_lens=[900, 2048, 77], k_lens=[1500, 2048, 300], hq=8, hk=2, d=128, qbs=64, kbs=128,
+                     keep=0.4, diag=True, causal=True, scale=None, dtype=torch.float32)
+    out = _run(w)
+    assert out.dtype == torch.float32
+    assert_close_to_oracle(out, oracle_for(w), "fp32 medium")
+    assert torch.equal(out, _run(w))
+
+
+@pytest.mark.parametrize("q_mag,k_mag,v_mag", [(1e-6, 1e3, 1e-9), (3e4, 1e-4, 1e12), (1.0, 1.0, 1e-30)])
+def test_fp32_inputs_keep_their_range(q_mag, k_mag, v_mag):
+    # magnitudes that overflow or vanish in a plain 16-bit cast: the per-tensor power-of-two scaling must absorb them
+    w = make_problem(seed=32, q_lens=[300, 200], k_lens=[300, 333], hq=4, hk=2, d=64, qbs=32, kbs=48, keep=0.6, diag=True,
+                     causal=True, scale=None, dtype=torch.float32)
+    base = oracle_for(w)
+    w.q.mul_(q_mag); w.k.mul_(k_mag); w.v.mul_(v_mag)
+    w.softmax_scale = (64 ** -0.5) / (q_mag * k_mag)          # the same logits as the unscaled problem
+    out = _run(w).double().cpu() / v_mag
+    sel = ~torch.isnan(base)
+    err = (out[sel] - base.double()[sel]).abs()
+    assert err.max().item() <= 4e-3 and err.mean().item() <= 3e-4, (err.max().item(), err.mean().item())
+
+
+def test_fp32_strided_inputs_headdim_padding_and_zero_tensor():
+    w = make_problem(seed=33, q_lens=[130, 70], k_lens=[130, 90], hq=4, hk=2, d=18, qbs=32, kbs=16, keep=0.7, diag=True,
+                     causal=False, scale=0.3, dtype=torch.float32)
+    ref = oracle_for(w)
+    assert_close_to_oracle(_run(w), ref, "fp32 d=18")
+    wide = torch.randn(w.k.shape[0], 2, 40, device="cuda")
+    wide[:, :, 4:22] = w.k
+    w.k = wide[:, :, 4:22]                                       # rows not 16-byte aligned
+    assert_close_to_oracle(_run(w), ref, "fp32 strided")
+    w.v = torch.zeros_like(w.v)
+    assert torch.count_nonzero(_run(w)) == 0
+
+
+def test_fp32_through_the_combined_c_entry_point():
+    w = make_problem(seed=34, q_lens=[500, 64], k_lens=[700, 64], hq=4, hk=4, d=32, qbs=48, kbs=80, keep=0.5, diag=True,
+                     causal=True, scale=None, dtype=torch.float32)
+    rc, out, _ = _call_hbsa_fwd(w)
+    assert rc == 0
+    assert torch.equal(out, _run(w))
+    assert_close_to_oracle(out, oracle_for(w), "hbsa_fwd fp32")
