@@ -48,6 +48,9 @@ def load() -> ctypes.CDLL:
     lib.hbsa_fwd_prepare.argtypes = [vp] * 7 + [ctypes.c_size_t] + [ctypes.c_int32] * 7 + [i64p, vp]
     lib.hbsa_fwd_run.restype = ctypes.c_int
     lib.hbsa_fwd_run.argtypes = [vp] * 5 + [ctypes.c_size_t] + [ctypes.c_int32] * 11 + [ctypes.c_float, i64p, vp]
+    lib.hbsa_fwd_run_lse.restype = ctypes.c_int
+    lib.hbsa_fwd_run_lse.argtypes = ([vp] * 5 + [i64p, vp, ctypes.c_size_t] + [ctypes.c_int32] * 11
+                                     + [ctypes.c_float, i64p, vp])
     _lib = lib
     return lib
 

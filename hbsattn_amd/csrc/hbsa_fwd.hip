@@ -94,6 +94,8 @@ struct FwdParams {
   int32_t f32;    // fp32 inputs staged as fp16: the setup kernel derives the constants from the maxima
   int32_t nhead_k;
   struct Sched *sched;
+  float *lse;             // optional [total_q, nhead_q] log-sum-exp output (nullptr: none)
+  int64_t lse_s, lse_h;   // its strides in elements
 };
 
 // --------------------------------------------------------------------------------------
@@ -955,6 +957,12 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     if (active) {
       const float l_tot = half_sum(l_run);
       const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+      if (p.lse != nullptr && g32 == 0 && l32 < nrows) {
+        // natural-log sum over the row's visible keys of exp(scale * q.k); m_run is the (possibly
+        // lagging) reference maximum the row sum was accumulated under, which makes this exact
+        const float lse = l_tot > 0.f ? (m_run * sm_c + __builtin_amdgcn_logf(l_tot)) * 0.69314718055994531f : -INFINITY;
+        p.lse[(int64_t)(row_begin + row0 + l32) * p.lse_s + (int64_t)hq * p.lse_h] = lse;
+      }
       if (l32 < nrows) {
         char *orow = p.out + (int64_t)(row_begin + row0 + l32) * p.o_s + (int64_t)hq * p.o_h;
         if constexpr (OUT32) {
@@ -1146,7 +1154,18 @@ int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out, void *w
                  int32_t dtype, int32_t total_q, int32_t total_k, int32_t nhead_q, int32_t nhead_k, int32_t headdim,
                  int32_t num_q_block, int32_t num_k_block, int32_t q_block_size, int32_t k_block_size, int32_t causal,
                  float softmax_scale, const int64_t *strides, void *stream) {
+  return hbsa_fwd_run_lse(q, k, v, out, nullptr, nullptr, workspace, workspace_bytes, dtype, total_q, total_k, nhead_q,
+                          nhead_k, headdim, num_q_block, num_k_block, q_block_size, k_block_size, causal, softmax_scale,
+                          strides, stream);
+}
+
+int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, float *lse, const int64_t *lse_strides,
+                     void *workspace, size_t workspace_bytes, int32_t dtype, int32_t total_q, int32_t total_k,
+                     int32_t nhead_q, int32_t nhead_k, int32_t headdim, int32_t num_q_block, int32_t num_k_block,
+                     int32_t q_block_size, int32_t k_block_size, int32_t causal, float softmax_scale,
+                     const int64_t *strides, void *stream) {
   g_err[0] = 0;
+  if (lse != nullptr && lse_strides == nullptr) return fail(HBSA_ERR_INVALID_ARGUMENT, "lse without lse_strides");
   if (total_q < 0 || total_k < 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "negative size");
   if (total_q == 0 || num_q_block == 0 || nhead_q == 0) return 0;  // nothing to write
   if (!q || !k || !v || !out || !workspace || !strides) return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer argument");
@@ -1180,6 +1199,9 @@ int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out, void *w
   fp.sched = (Sched *)((char *)workspace + sched_offset(num_q_block));
   fp.nhead_k = nhead_k;
   fp.f32 = f32 ? 1 : 0;
+  fp.lse = lse;
+  fp.lse_s = lse ? lse_strides[0] : 0;
+  fp.lse_h = lse ? lse_strides[1] : 0;
   if (f32) {
     // fp16 staging copies (contiguous) behind the bit words; the attention kernel reads those
     char *sq = (char *)workspace + base;

@@ -90,8 +90,10 @@ def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_s
     return PreparedMask(workspace, nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, causal)
 
 
-def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale) -> torch.Tensor:
-    """Runs the attention kernel (``hbsa_fwd_run``) on the current stream from a prepared mask."""
+def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = False):
+    """Runs the attention kernel (``hbsa_fwd_run`` / ``hbsa_fwd_run_lse``) on the current stream from a
+    prepared mask.  With ``return_lse`` the result is ``(out, lse)``, ``lse`` a float32
+    ``[total_q, nhead_q]`` tensor: log of the sum over a row's visible keys of exp(scale * q.k)."""
     if not q.is_cuda:
         raise RuntimeError("hbsattn_amd runs on MI355X only: q/k/v must be CUDA(HIP) tensors; there is no CPU path")
     if not (k.device == q.device and v.device == q.device and prepared.workspace.device == q.device):
@@ -115,8 +117,9 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale) -> torch.Tensor:
 
     lib = _lib.load()
     out = torch.empty((total_q, nhead_q, headdim), dtype=q.dtype, device=q.device)
+    lse = torch.empty((total_q, nhead_q), dtype=torch.float32, device=q.device) if return_lse else None
     if total_q == 0:
-        return out
+        return (out, lse) if return_lse else out
     d_run = next(d for d in _NATIVE_HEADDIMS if d >= headdim)
     if d_run != headdim:  # zero columns add nothing to q.k and give zero output columns
         q, k, v = _pad_headdim(q, d_run), _pad_headdim(k, d_run), _pad_headdim(v, d_run)
@@ -137,17 +140,19 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale) -> torch.Tensor:
             grown[: ws.numel()].copy_(ws)
             prepared.workspace = ws = grown
     with torch.cuda.device(q.device):
-        rc = lib.hbsa_fwd_run(q.data_ptr(), k.data_ptr(), v.data_ptr(), out_run.data_ptr(), ws.data_ptr(), ws.numel(),
-                              _DTYPE_CODES[q.dtype], total_q, total_k, nhead_q, nhead_k, d_run, prepared.num_q_block,
-                              prepared.num_k_block, prepared.q_block_size, prepared.k_block_size, int(prepared.causal),
-                              scale, strides, torch.cuda.current_stream().cuda_stream)
+        lse_strides = (ctypes.c_int64 * 2)(*lse.stride()) if return_lse else None
+        rc = lib.hbsa_fwd_run_lse(q.data_ptr(), k.data_ptr(), v.data_ptr(), out_run.data_ptr(),
+                                  lse.data_ptr() if return_lse else None, lse_strides, ws.data_ptr(), ws.numel(),
+                                  _DTYPE_CODES[q.dtype], total_q, total_k, nhead_q, nhead_k, d_run, prepared.num_q_block,
+                                  prepared.num_k_block, prepared.q_block_size, prepared.k_block_size,
+                                  int(prepared.causal), scale, strides, torch.cuda.current_stream().cuda_stream)
     if rc != 0:
         raise RuntimeError(f"hbsa_fwd_run failed (code {rc}): {_lib.last_error()}")
     # The launch is queued on the current stream; torch's caching allocator keeps padded copies
     # alive until work queued on that stream before their release has run.
     if out_run is not out:
         out.copy_(out_run[:, :, :headdim])
-    return out
+    return (out, lse) if return_lse else out
 
 
 def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, softmax_scale,

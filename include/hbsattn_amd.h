@@ -146,6 +146,25 @@ int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out,
                  int32_t causal, float softmax_scale,
                  const int64_t *strides, void *stream);
 
+/*
+ * hbsa_fwd_run that also writes, per query row and q head, the natural logarithm of the sum over
+ * the row's visible keys of exp(softmax_scale * q.k) (-inf for a row without visible keys):
+ * what merging attention over disjoint key sets needs.  The reference computes a per-row
+ * `lse` scratch but without the running maximum and does not return it
+ * (reference hbsattn/fwd_triton_auto_tile_size.py:246-251, 273, 310); this is the complete value.
+ *   lse           float [total_q, nhead_q] with element strides lse_strides = { tok, head };
+ *                 NULL = same as hbsa_fwd_run
+ */
+int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out,
+                     float *lse, const int64_t *lse_strides,
+                     void *workspace, size_t workspace_bytes,
+                     int32_t dtype, int32_t total_q, int32_t total_k,
+                     int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+                     int32_t num_q_block, int32_t num_k_block,
+                     int32_t q_block_size, int32_t k_block_size,
+                     int32_t causal, float softmax_scale,
+                     const int64_t *strides, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -85,14 +85,16 @@ def hbsa_oracle(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                 block_mask: torch.Tensor, q_block_size: int, k_block_size: int,
                 causal: bool, softmax_scale: Optional[float],
                 *, q_rows: Optional[Iterable[int]] = None, q_heads: Optional[Iterable[int]] = None,
-                compute_dtype: torch.dtype = torch.float32, row_chunk: int = 2048) -> torch.Tensor:
+                compute_dtype: torch.dtype = torch.float32, row_chunk: int = 2048, return_lse: bool = False):
     """Masked-dense block-sparse attention forward on CPU tensors.
 
     ``q [total_q, Hq, D]``, ``k, v [total_k, Hk, D]`` (any float dtype, upcast to
     ``compute_dtype``), ``block_mask [Hk, num_q_block, num_k_block]`` over *global*
     block indices.  Returns ``compute_dtype`` output of shape ``[total_q, Hq, D]``;
     with ``q_rows`` / ``q_heads`` only those rows / heads are computed, the rest is
-    NaN so an accidental comparison against an uncomputed entry fails.
+    NaN so an accidental comparison against an uncomputed entry fails.  With ``return_lse`` the
+    result is ``(out, lse)``, ``lse [total_q, Hq]`` = natural-log sum of exp(scaled scores) over a
+    row's visible keys (-inf for a row without any), NaN where not computed.
     """
     cu_q = [int(x) for x in cu_q_seqlens]
     cu_k = [int(x) for x in cu_k_seqlens]
@@ -109,6 +111,7 @@ def hbsa_oracle(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
 
     partial = q_rows is not None or q_heads is not None
     out = torch.full((total_q, hq, d), float("nan") if partial else 0.0, dtype=compute_dtype)
+    lse = torch.full((total_q, hq), float("nan") if partial else float("-inf"), dtype=compute_dtype)
     heads = sorted(set(int(h) for h in q_heads)) if q_heads is not None else list(range(hq))
     row_sel = None
     if q_rows is not None:
@@ -147,7 +150,8 @@ def hbsa_oracle(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                     p = torch.softmax(s, dim=1)
                     p = torch.nan_to_num(p, nan=0.0)  # rows with no visible key -> exactly 0
                     out[qs + rows, h] = p @ vb
-    return out
+                    lse[qs + rows, h] = torch.logsumexp(s, dim=1)
+    return (out, lse) if return_lse else out
 
 
 # --------------------------------------------------------------------------- #

@@ -343,3 +343,48 @@ def test_fp32_through_the_combined_c_entry_point():
     assert rc == 0
     assert torch.equal(out, _run(w))
     assert_close_to_oracle(out, oracle_for(w), "hbsa_fwd fp32")
+
+
+# ---------------------------------------------------------------------------------------
+# log-sum-exp output
+# ---------------------------------------------------------------------------------------
+def _run_lse(w, mask=None):
+    from hbsattn_amd.interface import hbsa_prepare, hbsa_run
+    prepared = hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask if mask is None else mask, w.q_block_size,
+                            w.k_block_size, w.causal, w.q_meta[0], w.q_meta[2], w.q_meta[3], w.k_meta[0], w.k_meta[3])
+    out, lse = hbsa_run(w.q, w.k, w.v, prepared, w.softmax_scale, return_lse=True)
+    torch.cuda.synchronize()
+    return out, lse
+
+
+@pytest.mark.parametrize("dtype,scale", [(torch.bfloat16, None), (torch.float16, -0.3), (torch.float32, 0.2)])
+def test_lse_matches_oracle(dtype, scale):
+    w = make_problem(seed=41, q_lens=[700, 90, 1024], k_lens=[300, 90, 2048], hq=8, hk=2, d=64, qbs=48, kbs=80, keep=0.4,
+                     diag=False, causal=True, scale=scale, dtype=dtype)
+    out, lse = _run_lse(w)
+    ref_out, ref_lse = hbsa_oracle(w.q.cpu(), w.k.cpu(), w.v.cpu(), w.cu_q, w.cu_k, w.block_mask.cpu(), w.q_block_size,
+                                   w.k_block_size, w.causal, w.softmax_scale, return_lse=True)
+    assert torch.equal(out, _run(w))                          # asking for lse does not change out
+    assert_close_to_oracle(out, ref_out, "lse run")
+    lse = lse.cpu()
+    no_keys = torch.isinf(ref_lse)
+    assert no_keys.any() and torch.equal(torch.isinf(lse) & (lse < 0), no_keys)
+    # scores are fp32 sums of exact products of the 16-bit inputs; fp32 inputs carry 11-bit operands
+    tol = 5e-3 if dtype == torch.float32 else 2e-3
+    assert (lse[~no_keys] - ref_lse[~no_keys]).abs().max().item() <= tol
+
+
+def test_lse_merges_two_runs_over_disjoint_key_blocks():
+    w = make_problem(seed=42, q_lens=[2048, 1000], k_lens=[2048, 1500], hq=4, hk=4, d=128, qbs=128, kbs=128, keep=0.5,
+                     diag=True, causal=True, scale=None)
+    full, lse = _run_lse(w)
+    part_a = w.block_mask.clone(); part_a[:, :, 1::2] = False
+    part_b = w.block_mask.clone(); part_b[:, :, 0::2] = False
+    oa, la = _run_lse(w, part_a)
+    ob, lb = _run_lse(w, part_b)
+    merged = torch.logaddexp(la, lb)
+    assert (merged - lse).abs().max().item() <= 1e-4
+    wa = torch.nan_to_num(torch.exp(la - merged), nan=0.0).unsqueeze(-1)
+    wb = torch.nan_to_num(torch.exp(lb - merged), nan=0.0).unsqueeze(-1)
+    err = (wa * oa.float() + wb * ob.float() - full.float()).abs()
+    assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3

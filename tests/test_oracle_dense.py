@@ -162,3 +162,40 @@ def test_dense_partial_rows_and_heads():
     for r in (3, 39, 40, 99):
         torch.testing.assert_close(part[r, [1, 2]], full[r, [1, 2]], atol=1e-6, rtol=1e-6)
     assert torch.isnan(part[0]).all() and torch.isnan(part[3, 0]).all()
+
+
+# ---------------------------------------------------------------------------------------
+# log-sum-exp output of the oracle
+# ---------------------------------------------------------------------------------------
+def test_lse_equals_library_logsumexp_on_dense_and_causal_cases():
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(n, 2, 16, generator=g) for n in (48, 80, 80))
+    mask = torch.ones(2, 3, 5, dtype=torch.bool)
+    out, lse = hbsa_oracle(q, k, v, [0, 48], [0, 80], mask, 16, 16, False, 0.4, return_lse=True)
+    s = torch.einsum("qhd,khd->hqk", q, k) * 0.4
+    assert torch.allclose(lse, torch.logsumexp(s, -1).T, atol=1e-5)
+    assert torch.allclose(out, torch.einsum("hqk,khd->qhd", torch.softmax(s, -1), v), atol=1e-5)
+    out_c, lse_c = hbsa_oracle(q, k, v, [0, 48], [0, 80], mask, 16, 16, True, 0.4, return_lse=True)
+    vis = torch.ones(48, 80, dtype=torch.bool).tril(diagonal=80 - 48)
+    assert torch.allclose(lse_c, torch.logsumexp(s.masked_fill(~vis, float("-inf")), -1).T, atol=1e-5)
+
+
+def test_lse_merges_attention_over_disjoint_key_sets_and_is_minus_inf_without_keys():
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(64, 4, 8, generator=g)
+    k, v = (torch.randn(96, 2, 8, generator=g) for _ in range(2))
+    cu_q, cu_k = [0, 40, 64], [0, 30, 96]
+    mask = torch.rand(2, 5, 7, generator=g) < 0.6
+    part_a = mask.clone(); part_a[:, :, 1::2] = False
+    part_b = mask.clone(); part_b[:, :, 0::2] = False
+    full, lse = hbsa_oracle(q, k, v, cu_q, cu_k, mask, 16, 16, True, None, return_lse=True)
+    oa, la = hbsa_oracle(q, k, v, cu_q, cu_k, part_a, 16, 16, True, None, return_lse=True)
+    ob, lb = hbsa_oracle(q, k, v, cu_q, cu_k, part_b, 16, 16, True, None, return_lse=True)
+    merged_lse = torch.logaddexp(la, lb)
+    assert torch.allclose(merged_lse, lse, atol=1e-5, equal_nan=True)
+    wa = torch.nan_to_num(torch.exp(la - merged_lse), nan=0.0).unsqueeze(-1)
+    wb = torch.nan_to_num(torch.exp(lb - merged_lse), nan=0.0).unsqueeze(-1)
+    assert torch.allclose(wa * oa + wb * ob, full, atol=1e-5)
+    empty = torch.isinf(lse) & (lse < 0)
+    assert empty.any()                                      # causal rows of sequence 0 ahead of every key (q_len > k_len)
+    assert torch.equal(empty, (full == 0).all(-1))
