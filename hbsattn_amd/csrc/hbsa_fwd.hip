@@ -1100,6 +1100,33 @@ int hbsa_abi_version(void) { return HBSA_ABI_VERSION; }
 
 const char *hbsa_last_error(void) { return g_err; }
 
+int hbsa_calculate_blocks(const int32_t *cu_seqlen, int32_t batch, int32_t block_size, int32_t *num_block,
+                          int32_t *cu_num_block, int32_t *cu_block, int32_t *block_to_batch, int32_t capacity) {
+  g_err[0] = 0;
+  if (!cu_seqlen || !num_block || batch < 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer or negative batch");
+  if (block_size <= 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "block_size must be positive");
+  int64_t total = 0;
+  if (cu_num_block) cu_num_block[0] = 0;
+  for (int b = 0; b < batch; ++b) {
+    const int64_t len = (int64_t)cu_seqlen[b + 1] - cu_seqlen[b];
+    if (len < 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "cu_seqlen decreases at sequence %d", b);
+    total += (len + block_size - 1) / block_size;
+    if (total > 0x7fffffff) return fail(HBSA_ERR_UNSUPPORTED, "more than 2^31 - 1 blocks");
+    if (cu_num_block) cu_num_block[b + 1] = (int32_t)total;
+  }
+  *num_block = (int32_t)total;
+  if (!cu_block && !block_to_batch) return 0;
+  if (capacity < total) return fail(HBSA_ERR_WORKSPACE_TOO_SMALL, "capacity %d < %lld blocks", capacity, (long long)total);
+  int32_t j = 0;
+  if (cu_block) cu_block[0] = 0;
+  for (int b = 0; b < batch; ++b)
+    for (int64_t start = cu_seqlen[b]; start < cu_seqlen[b + 1]; start += block_size, ++j) {
+      if (block_to_batch) block_to_batch[j] = b;
+      if (cu_block) cu_block[j + 1] = (int32_t)std::min<int64_t>(start + block_size, cu_seqlen[b + 1]);
+    }
+  return 0;
+}
+
 size_t hbsa_fwd_workspace_bytes(int32_t nhead_k, int32_t num_q_block, int32_t num_k_block) {
   if (nhead_k <= 0 || num_q_block <= 0 || num_k_block <= 0) return 256;
   const size_t bits = align_up((size_t)nhead_k * num_q_block * words_per_row(num_k_block) * sizeof(uint32_t), 256);

@@ -48,6 +48,19 @@ int hbsa_abi_version(void);
 const char *hbsa_last_error(void);
 
 /*
+ * Block geometry of a packed variable-length batch, on the HOST (all pointers are host memory):
+ * the counterpart of hbsattn.utils.calculate_blocks (reference hbsattn/utils.py:7-50) for callers
+ * without torch.  Blocks restart at every sequence start and the last block of a sequence may be
+ * short.  Writes *num_block, cu_num_block[batch+1] (first global block of each sequence) and, when
+ * given, cu_block[num_block+1] (token boundaries; cu_block[0] = 0 like the reference, which
+ * assumes cu_seqlen[0] = 0) and block_to_batch[num_block]; `capacity` is the number of blocks the
+ * last two can hold.  Call it with cu_block = block_to_batch = NULL to size them first.
+ */
+int hbsa_calculate_blocks(const int32_t *cu_seqlen, int32_t batch, int32_t block_size,
+                          int32_t *num_block, int32_t *cu_num_block,
+                          int32_t *cu_block, int32_t *block_to_batch, int32_t capacity);
+
+/*
  * Bytes of device scratch hbsa_fwd needs for this problem.  Replaces the launcher's
  * own scratch allocations (reference hbsattn/fwd_triton_auto_tile_size.py:273-274:
  * `lse`, `tmp`); here the scratch holds the compacted work description the pre-pass

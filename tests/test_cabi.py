@@ -91,3 +91,52 @@ def test_empty_problem_is_a_no_op():
     lib = _lib.load()
     assert _call_fwd(lib, total_q=0, q=None) == 0
     assert _lib.last_error() == ""
+
+
+def _c_calculate_blocks(cu, block_size):
+    import numpy as np
+    lib = _lib.load()
+    cu = np.asarray(cu, dtype=np.int32)
+    batch = len(cu) - 1
+    nb = ctypes.c_int32(-1)
+    cu_nb = np.full(batch + 1, -1, dtype=np.int32)
+    rc = lib.hbsa_calculate_blocks(cu.ctypes.data, batch, block_size, ctypes.addressof(nb), cu_nb.ctypes.data, None, None, 0)
+    assert rc == 0, _lib.last_error()
+    cu_block = np.full(nb.value + 1, -1, dtype=np.int32)
+    b2b = np.full(nb.value, -1, dtype=np.int32)
+    rc = lib.hbsa_calculate_blocks(cu.ctypes.data, batch, block_size, ctypes.addressof(nb), cu_nb.ctypes.data,
+                                   cu_block.ctypes.data, b2b.ctypes.data, nb.value)
+    assert rc == 0, _lib.last_error()
+    return nb.value, cu_block.tolist(), b2b.tolist(), cu_nb.tolist()
+
+
+def test_host_calculate_blocks_matches_oracle_and_readme_example():
+    import random
+    from oracle.dense import calculate_blocks_oracle
+    # the reference's worked example (README.md:49-63 of the reference): last-block sizes 16, 13, 7, 2, 7
+    nb, cu_block, b2b, cu_nb = _c_calculate_blocks([0, 32, 61, 100, 134, 157], 16)
+    assert nb == 12 and cu_nb == [0, 2, 4, 7, 10, 12]
+    assert [cu_block[cu_nb[b + 1]] - cu_block[cu_nb[b + 1] - 1] for b in range(5)] == [16, 13, 7, 2, 7]
+    rng = random.Random(3)
+    for _ in range(50):
+        lens = [rng.randrange(0, 300) for _ in range(rng.randrange(0, 7))]
+        cu = [0]
+        for n in lens:
+            cu.append(cu[-1] + n)
+        bs = rng.choice([16, 32, 48, 80, 128])
+        got = _c_calculate_blocks(cu, bs)
+        ref = calculate_blocks_oracle(cu, bs)
+        assert got == (ref[0], list(ref[1]), list(ref[2]), list(ref[3])), (cu, bs)
+
+
+def test_host_calculate_blocks_rejects_bad_input():
+    import numpy as np
+    lib = _lib.load()
+    nb = ctypes.c_int32(0)
+    cu = np.asarray([0, 10, 5], dtype=np.int32)
+    assert lib.hbsa_calculate_blocks(cu.ctypes.data, 2, 16, ctypes.addressof(nb), None, None, None, 0) == -1
+    cu = np.asarray([0, 100], dtype=np.int32)
+    assert lib.hbsa_calculate_blocks(cu.ctypes.data, 1, 0, ctypes.addressof(nb), None, None, None, 0) == -1
+    small = np.zeros(3, dtype=np.int32)
+    assert lib.hbsa_calculate_blocks(cu.ctypes.data, 1, 16, ctypes.addressof(nb), None, small.ctypes.data, None, 2) == -3
+    assert nb.value == 7
