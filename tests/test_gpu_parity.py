@@ -388,3 +388,15 @@ def test_lse_merges_two_runs_over_disjoint_key_blocks():
     wb = torch.nan_to_num(torch.exp(lb - merged), nan=0.0).unsqueeze(-1)
     err = (wa * oa.float() + wb * ob.float() - full.float()).abs()
     assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3
+
+
+# ---------------------------------------------------------------------------------------
+# items longer than one tile list (1024 tiles) and mask rows longer than one 2048-block window
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("kbs,keep,causal", [(64, 1.0, False), (128, 0.9, True), (48, 1.0, False), (80, 0.7, True)])
+def test_very_long_key_sequences_refill_the_tile_list(kbs, keep, causal):
+    w = make_problem(seed=51, q_lens=[96, 40], k_lens=[150000, 3000], hq=2, hk=1, d=64, qbs=32, kbs=kbs, keep=keep, diag=True,
+                     causal=causal, scale=None)
+    out = _run(w)
+    assert_close_to_oracle(out, oracle_for(w), f"long keys kbs={kbs}")
+    assert torch.equal(out, _run(w))
