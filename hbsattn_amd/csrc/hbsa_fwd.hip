@@ -80,6 +80,22 @@ struct PrepParams {
   int32_t nqb, qbs, kbs, wpr, causal;
 };
 
+// Division by a launch constant d, exact for 0 <= n < 2^31: n / d == (n * m) >> s with
+// s = 31 + ceil(log2 d), m = ceil(2^s / d) (which fits 32 bits).  Three scalar instructions where
+// a hardware-less integer division takes about forty.
+struct FastDiv {
+  uint32_t m, s;
+};
+__host__ __device__ inline uint32_t fast_div(uint32_t n, FastDiv f) { return (uint32_t)(((uint64_t)n * f.m) >> f.s); }
+inline FastDiv make_fast_div(uint32_t d) {
+  uint32_t l = 0;
+  while (((uint64_t)1 << l) < d) ++l;
+  FastDiv f;
+  f.s = 31 + l;
+  f.m = (uint32_t)((((uint64_t)1 << f.s) + d - 1) / d);
+  return f;
+}
+
 struct FwdParams {
   const char *q, *k, *v;
   char *out;
@@ -91,6 +107,7 @@ struct FwdParams {
   int32_t nsub;   // workgroups per (kv head, q block) = ceil(ratio * wps / 4)
   uint32_t q_sign;  // 0x80008000 when softmax_scale < 0 (Q is negated, |scale| used)
   float c;        // |softmax_scale| * log2(e); the kernel reads the launch's value from sched
+  FastDiv div_nsub, div_nqb, div_kbs;   // divisions on the scheduler's path
   int32_t f32;    // fp32 inputs staged as fp16: the setup kernel derives the constants from the maxima
   int32_t nhead_k;
   struct Sched *sched;
@@ -320,7 +337,7 @@ __device__ __forceinline__ int pack_tile(int pos, int valid) { return ((pos >> 4
 // the item's tile sequence, written to list[0..); returns the item's total tile count.
 // Executed by one whole wavefront; `first_words`: lane i holds bit word i of the row.
 __device__ __forceinline__ int build_tile_list(int *list, int chunk_base, const uint32_t *row, int nwords, int kbs,
-                                                int kmax, uint32_t first_words, int lane) {
+                                                FastDiv div_kbs, int kmax, uint32_t first_words, int lane) {
   if (kmax <= 0 || nwords <= 0) return 0;
   int total = 0;
   if ((kbs & 63) == 0) {
@@ -330,7 +347,7 @@ __device__ __forceinline__ int build_tile_list(int *list, int chunk_base, const 
     // the tiles of the kept blocks below it.
     const int tpb = kbs >> 6;
     const int half = lane >> 5, bit = lane & 31;
-    const int j_last = (kmax - 1) / kbs;   // no bit above this block is set
+    const int j_last = (int)fast_div((uint32_t)(kmax - 1), div_kbs);   // no bit above this block is set
     int window = 0;
     uint32_t held = lane < nwords ? first_words : 0u;
     for (int w2 = 0; w2 < nwords; w2 += 2) {
@@ -499,10 +516,11 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     while (tries < 8) {
       const int v = (first_queue + tries) & 7;
       if (claimed < queue_len(v)) {
-        const uint32_t t = claimed / (uint32_t)p.nsub;
-        st_sub = (int)(claimed % (uint32_t)p.nsub);
-        st_hk = v + 8 * (int)(t / (uint32_t)p.nqb);
-        st_qb = p.nqb - 1 - (int)(t % (uint32_t)p.nqb);
+        const uint32_t t = fast_div(claimed, p.div_nsub);
+        st_sub = (int)(claimed - t * (uint32_t)p.nsub);
+        const uint32_t hq8 = fast_div(t, p.div_nqb);
+        st_hk = v + 8 * (int)hq8;
+        st_qb = p.nqb - 1 - (int)(t - hq8 * (uint32_t)p.nqb);
         break;
       }
       if (++tries >= 8) break;
@@ -525,7 +543,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
       const int nkblk = __builtin_amdgcn_readlane((int)st_info, 6);
       const int kmax = __builtin_amdgcn_readlane((int)st_info, 7);
       total = build_tile_list(lds_list + c * kListCap, 0, p.bits + ((size_t)st_hk * p.nqb + st_qb) * p.wpr,
-                              2 * ((nkblk + 63) >> 6), p.kbs, kmax, st_bits, lane);
+                              2 * ((nkblk + 63) >> 6), p.kbs, p.div_kbs, kmax, st_bits, lane);
     }
     if (lane == 0) {
       hdr[H_HK] = st_hk; hdr[H_QB] = st_qb; hdr[H_SUB] = st_sub; hdr[H_TOTAL] = total;
@@ -942,7 +960,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         const QBlockInfo inf = p.info[qb];
         const uint32_t *row = p.bits + ((size_t)cur_hk * p.nqb + qb) * p.wpr;
         const int nwords = 2 * ((inf.nkblk + 63) >> 6);
-        (void)build_tile_list(lds_list + c * kListCap, chunk_base, row, nwords, p.kbs, inf.kmax,
+        (void)build_tile_list(lds_list + c * kListCap, chunk_base, row, nwords, p.kbs, p.div_kbs, inf.kmax,
                               lane < nwords ? row[lane] : 0u, lane);
       }
       __syncthreads();
@@ -956,7 +974,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     // ---- epilogue: normalise, convert, store (rows with no visible key store exact zeros)
     if (active) {
       const float l_tot = half_sum(l_run);
-      const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+      const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;   // 1 ulp; a full division is ten instructions
       if (p.lse != nullptr && g32 == 0 && l32 < nrows) {
         // natural-log sum over the row's visible keys of exp(scale * q.k); m_run is the (possibly
         // lagging) reference maximum the row sum was accumulated under, which makes this exact
@@ -1253,6 +1271,9 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
   fp.causal = causal ? 1 : 0;
   fp.wps = (q_block_size + kWaveRows - 1) / kWaveRows;
   fp.nsub = (fp.ratio * fp.wps + 3) / 4;
+  fp.div_nsub = make_fast_div((uint32_t)fp.nsub);
+  fp.div_nqb = make_fast_div((uint32_t)num_q_block);
+  fp.div_kbs = make_fast_div((uint32_t)k_block_size);
   fp.q_sign = softmax_scale < 0.f ? 0x80008000u : 0u;
   float c = std::fabs(softmax_scale) * kLog2e;
   if (c < 1e-30f) c = 1e-30f;  // scale 0: uniform weights over the visible keys, and -inf * c stays -inf
