@@ -35,5 +35,25 @@ def build(verbose: bool = False) -> str:
     return OUTPUT
 
 
+EXAMPLE_SOURCE = os.path.join(_HERE, "csrc", "cabi_example.cpp")
+EXAMPLE_OUTPUT = os.path.join(_HERE, "cabi_example")
+
+
+def build_example(verbose: bool = False) -> str:
+    """The torch-free C++ caller of the library (``csrc/cabi_example.cpp``); run it on a GPU box as
+    ``./hbsattn_amd/cabi_example``."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    cmd = [hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I" + os.path.join(_ROOT, "include"), EXAMPLE_SOURCE,
+           "-L" + _HERE, "-lhbsattn_amd", "-Wl,-rpath,$ORIGIN", "-o", EXAMPLE_OUTPUT]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+        raise RuntimeError("hipcc failed: " + " ".join(cmd))
+    if verbose:
+        print(" ".join(cmd))
+    return EXAMPLE_OUTPUT
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_example(verbose=True))
