@@ -11,6 +11,7 @@ ABI_VERSION = 2
 DTYPE_BF16 = 0
 DTYPE_F16 = 1
 DTYPE_F32 = 2
+DTYPE_F32_STAGED16 = 3
 
 _lib = None
 

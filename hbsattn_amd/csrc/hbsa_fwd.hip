@@ -1110,6 +1110,176 @@ int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
   return 0;
 }
 
+
+// --------------------------------------------------------------------------------------
+// fp32 kernel: fp32 operands, fp32 MFMA (v_mfma_f32_32x32x2_f32), fp32 softmax and output, for
+// callers that need the arithmetic of the reference's fp32 path (dot products without operand
+// rounding, reference hbsattn/fwd_triton_auto_tile_size.py:205,225).  One workgroup per work item
+// (kv head, q block, group of four wave slots), no persistence or prefetching: the fp32 matrix
+// rate (a sixteenth of the bf16 one) bounds it, not the loads.
+//
+// Same operand roles as the 16-bit kernel: S^T = K.Q^T with K rows from LDS and Q^T in registers,
+// O^T += V^T.P^T with P^T taken from the S^T accumulator in place.  A 32x32x2 MFMA contracts over
+// two indices, one per half of the wavefront; which two is free as long as both operands agree:
+//   S: step (j, e), half g contracts over d = 8*j + 4*g + e, so a lane reads 4 consecutive floats of
+//      its K row per j (one ds_read_b128) and holds Q the same way;
+//   PV: step i, half g contracts over key 8*(i/4) + 4*g + (i%4), which is exactly the key whose
+//      score the lane holds in accumulator element i.
+// LDS: K[64][D+4] and V[64][D+4] floats (the 4-float pad spreads the rows over the banks).
+// --------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_f32_kernel(FwdParams p, float c_signed) {
+  constexpr int LD = D + 4;       // LDS row stride in floats
+  constexpr int DJ = D / 8;       // ds_read_b128 steps of S
+  constexpr int DT = D / 32;      // 32-row tiles of O^T
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  float *lds_k = (float *)lds_raw;
+  float *lds_v = lds_k + kTileKeys * LD;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g32 = lane >> 5, l32 = lane & 31;
+
+  // item: heaviest q blocks first, like the queues of the 16-bit kernel
+  const uint32_t t = fast_div(blockIdx.x, p.div_nsub);
+  const int sub = (int)(blockIdx.x - t * (uint32_t)p.nsub);
+  const uint32_t hk_u = fast_div(t, p.div_nqb);
+  const int hk = (int)hk_u;
+  const int qb = p.nqb - 1 - (int)(t - hk_u * (uint32_t)p.nqb);
+  const QBlockInfo inf = p.info[qb];
+
+  const int slot = sub * 4 + wave;
+  const int head_in_group = slot / p.wps;
+  const int row0 = (slot % p.wps) * kWaveRows;
+  const int nrows = min(kWaveRows, inf.rows - row0);
+  const bool active = head_in_group < p.ratio && nrows > 0;
+  const int hq = hk * p.ratio + head_in_group;
+
+  // Q^T fragments, pre-multiplied by softmax_scale * log2(e): scores come out in log2 units
+  f32x4 qf[DJ];
+  {
+    const int r = min(row0 + l32, inf.rows - 1);
+    const char *qrow = p.q + (int64_t)(inf.row_begin + r) * p.q_s + (int64_t)hq * p.q_h;
+#pragma unroll
+    for (int j = 0; j < DJ; ++j) {
+      f32x4 x = {0.f, 0.f, 0.f, 0.f};
+      if (active) x = *(const f32x4 *)(qrow + (8 * j + 4 * g32) * 4);
+      qf[j] = x * c_signed;
+    }
+  }
+  f32x16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const int lane_kvis = inf.q_pos + min(row0 + l32, inf.rows - 1) + inf.shift;   // last key position this query sees
+  const int wave_kvis_max = inf.q_pos + row0 + nrows - 1 + inf.shift;
+  const char *kg = p.k + (int64_t)hk * p.k_h + (int64_t)inf.key_begin * p.k_s;
+  const char *vg = p.v + (int64_t)hk * p.v_h + (int64_t)inf.key_begin * p.v_s;
+  const uint32_t *bits = p.bits + ((size_t)hk * p.nqb + qb) * p.wpr;
+  const int nwords = inf.kmax > 0 ? (inf.nkblk + 31) >> 5 : 0;
+
+  for (int w = 0; w < nwords; ++w) {
+    uint32_t word = (uint32_t)__builtin_amdgcn_readfirstlane((int)bits[w]);
+    while (word != 0) {
+      const int j = w * 32 + __builtin_ctz(word);
+      word &= word - 1;
+      const int end = min(min((j + 1) * p.kbs, inf.klen), inf.kmax);
+      for (int pos = j * p.kbs; pos < end; pos += kTileKeys) {   // ---- one tile of up to 64 keys
+        const int valid = min(kTileKeys, end - pos);
+        __syncthreads();   // the previous tile has been consumed
+        for (int idx = threadIdx.x; idx < kTileKeys * (D / 4); idx += kThreads) {
+          const int r = idx / (D / 4), c4 = idx % (D / 4);
+          const int64_t tok = pos + min(r, valid - 1);   // rows past the end repeat the last one (masked below)
+          *(f32x4 *)(lds_k + r * LD + c4 * 4) = *(const f32x4 *)(kg + tok * p.k_s + c4 * 16);
+          *(f32x4 *)(lds_v + r * LD + c4 * 4) = *(const f32x4 *)(vg + tok * p.v_s + c4 * 16);
+        }
+        __syncthreads();
+        if (!active || (p.causal && pos > wave_kvis_max)) continue;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {   // ---- 32 keys at a time
+          if (32 * h >= valid || (p.causal && pos + 32 * h > wave_kvis_max)) continue;
+          f32x16 sc;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+          const float *krow = lds_k + (32 * h + l32) * LD + 4 * g32;
+#pragma unroll
+          for (int jj = 0; jj < DJ; ++jj) {
+            const f32x4 kv = *(const f32x4 *)(krow + 8 * jj);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[e], qf[jj][e], sc, 0, 0, 0);
+          }
+          int lim = valid - 32 * h;                                  // keys of this half below lim are visible
+          if (p.causal) lim = min(lim, lane_kvis - pos - 32 * h + 1);
+          float mx = -INFINITY;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            if (8 * (i >> 2) + 4 * g32 + (i & 3) >= lim) sc[i] = -INFINITY;
+            mx = fmaxf(mx, sc[i]);
+          }
+          mx = half_max(mx);
+          // no branch on per-query values here: the MFMAs below need every lane
+          const float m_new = fmaxf(m_run, mx);
+          const float m_ref = m_new == -INFINITY ? 0.f : m_new;       // a query that has seen no key yet
+          const float alpha = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - m_ref);
+          l_run *= alpha;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+          m_run = m_new;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            sc[i] = __builtin_amdgcn_exp2f(sc[i] - m_ref);
+            l_run += sc[i];
+          }
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const float *vrow = lds_v + (32 * h + 8 * (i >> 2) + 4 * g32 + (i & 3)) * LD + l32;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * dt], sc[i], o[dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+
+  if (!active) return;
+  const float l_tot = half_sum(l_run);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (l32 >= nrows) return;
+  const int64_t row = inf.row_begin + row0 + l32;
+  if (p.lse != nullptr && g32 == 0)
+    p.lse[row * p.lse_s + (int64_t)hq * p.lse_h] =
+        l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * 0.69314718055994531f : -INFINITY;
+  char *orow = p.out + row * p.o_s + (int64_t)hq * p.o_h;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      f32x4 wv = {o[dt][4 * i4 + 0] * inv, o[dt][4 * i4 + 1] * inv, o[dt][4 * i4 + 2] * inv, o[dt][4 * i4 + 3] * inv};
+      *(f32x4 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 4) = wv;
+    }
+}
+
+template <int D>
+int launch_fwd_f32(const FwdParams &fp, float c_signed, long long items, hipStream_t stream) {
+  constexpr int lds_bytes = 2 * kTileKeys * (D + 4) * 4;
+  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_f32_kernel<D>);
+  static thread_local bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  hipLaunchKernelGGL((hbsa_fwd_f32_kernel<D>), dim3((unsigned)items), dim3(kThreads), lds_bytes, stream, fp, c_signed);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail((int)e, "hbsa_fwd_f32_kernel launch: %s", hipGetErrorString(e));
+  return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1154,7 +1324,7 @@ size_t hbsa_fwd_workspace_bytes(int32_t nhead_k, int32_t num_q_block, int32_t nu
 size_t hbsa_fwd_workspace_bytes_dtype(int32_t dtype, int32_t total_q, int32_t total_k, int32_t nhead_q,
                                       int32_t nhead_k, int32_t headdim, int32_t num_q_block, int32_t num_k_block) {
   size_t n = hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block);
-  if (dtype == HBSA_DTYPE_F32 && total_q > 0 && total_k > 0 && nhead_q > 0 && nhead_k > 0 && headdim > 0)
+  if (dtype == HBSA_DTYPE_F32_STAGED16 && total_q > 0 && total_k > 0 && nhead_q > 0 && nhead_k > 0 && headdim > 0)
     n += f32_stage_bytes(total_q, nhead_q, headdim) + 2 * f32_stage_bytes(total_k, nhead_k, headdim);
   return n;
 }
@@ -1221,12 +1391,13 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
                 q_block_size, k_block_size);
   if (headdim != 32 && headdim != 64 && headdim != 128)
     return fail(HBSA_ERR_UNSUPPORTED, "headdim %d not in {32, 64, 128}", headdim);
-  if (dtype != HBSA_DTYPE_BF16 && dtype != HBSA_DTYPE_F16 && dtype != HBSA_DTYPE_F32)
+  if (dtype < HBSA_DTYPE_BF16 || dtype > HBSA_DTYPE_F32_STAGED16)
     return fail(HBSA_ERR_UNSUPPORTED, "dtype code %d not supported", dtype);
   if (num_k_block <= 0 || total_k <= 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "no keys");
   if (!std::isfinite(softmax_scale)) return fail(HBSA_ERR_INVALID_ARGUMENT, "softmax_scale is not finite");
-  const bool f32 = dtype == HBSA_DTYPE_F32;
-  if (int rc = check_strides(strides, f32)) return rc;
+  const bool f32 = dtype == HBSA_DTYPE_F32_STAGED16;    // fp32 tensors staged as scaled fp16
+  const bool f32_exact = dtype == HBSA_DTYPE_F32;       // fp32 tensors, fp32 MFMA
+  if (int rc = check_strides(strides, f32 || f32_exact)) return rc;
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
     return fail(HBSA_ERR_INVALID_ARGUMENT, "q/k/v/out must be 16-byte aligned");
   if ((uintptr_t)workspace & 255) return fail(HBSA_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
@@ -1264,8 +1435,9 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
     fp.v_s = fp.k_s; fp.v_h = fp.k_h;
     fp.o_s = strides[6] * 4; fp.o_h = strides[7] * 4;
   } else {
-    fp.q_s = strides[0] * 2; fp.q_h = strides[1] * 2; fp.k_s = strides[2] * 2; fp.k_h = strides[3] * 2;
-    fp.v_s = strides[4] * 2; fp.v_h = strides[5] * 2; fp.o_s = strides[6] * 2; fp.o_h = strides[7] * 2;
+    const int64_t es = f32_exact ? 4 : 2;
+    fp.q_s = strides[0] * es; fp.q_h = strides[1] * es; fp.k_s = strides[2] * es; fp.k_h = strides[3] * es;
+    fp.v_s = strides[4] * es; fp.v_h = strides[5] * es; fp.o_s = strides[6] * es; fp.o_h = strides[7] * es;
   }
   fp.nqb = num_q_block; fp.ratio = nhead_q / nhead_k; fp.kbs = k_block_size; fp.wpr = words_per_row(num_k_block);
   fp.causal = causal ? 1 : 0;
@@ -1281,6 +1453,14 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
   const long long items = (long long)nhead_k * num_q_block * fp.nsub;
   if (items > 0x7fffffffLL) return fail(HBSA_ERR_UNSUPPORTED, "too many work items (%lld)", items);
 
+  if (f32_exact) {
+    const float c_signed = softmax_scale * kLog2e;
+    switch (headdim) {
+      case 32: return launch_fwd_f32<32>(fp, c_signed, items, st);
+      case 64: return launch_fwd_f32<64>(fp, c_signed, items, st);
+      default: return launch_fwd_f32<128>(fp, c_signed, items, st);
+    }
+  }
   if (f32) {
     // setup (multipliers from the maxima), staging, attention: the launch order on the stream is the
     // dependency order
@@ -1321,12 +1501,12 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32
     return fail(HBSA_ERR_INVALID_ARGUMENT, "nhead_q (%d) must be divisible by nhead_k (%d)", nhead_q, nhead_k);
   if (headdim != 32 && headdim != 64 && headdim != 128)
     return fail(HBSA_ERR_UNSUPPORTED, "headdim %d not in {32, 64, 128}", headdim);
-  if (dtype != HBSA_DTYPE_BF16 && dtype != HBSA_DTYPE_F16 && dtype != HBSA_DTYPE_F32)
+  if (dtype < HBSA_DTYPE_BF16 || dtype > HBSA_DTYPE_F32_STAGED16)
     return fail(HBSA_ERR_UNSUPPORTED, "dtype code %d not supported", dtype);
   if (!std::isfinite(softmax_scale)) return fail(HBSA_ERR_INVALID_ARGUMENT, "softmax_scale is not finite");
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
     return fail(HBSA_ERR_INVALID_ARGUMENT, "q/k/v/out must be 16-byte aligned");
-  if (int rc = check_strides(strides, dtype == HBSA_DTYPE_F32)) return rc;
+  if (int rc = check_strides(strides, dtype == HBSA_DTYPE_F32 || dtype == HBSA_DTYPE_F32_STAGED16)) return rc;
   {
     const size_t need = hbsa_fwd_workspace_bytes_dtype(dtype, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
                                                        num_k_block);

@@ -10,6 +10,7 @@ that relies on it behaves the same.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional
 
 import torch
@@ -19,6 +20,29 @@ from .utils import calculate_blocks
 
 _NATIVE_HEADDIMS = (32, 64, 128)
 _DTYPE_CODES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16, torch.float32: _lib.DTYPE_F32}
+
+# How fp32 q/k/v are multiplied: "exact" = fp32 matrix instructions, the arithmetic of the reference's
+# fp32 path (``tl.dot(..., allow_tf32=False)``, reference hbsattn/fwd_triton_auto_tile_size.py:205,225);
+# "fast" = scaled fp16 staging copies and the 16-bit kernel (11-bit operand significands, about ten
+# times faster).  The environment variable HBSATTN_AMD_FP32_MODE sets the initial mode.
+_fp32_mode = os.environ.get("HBSATTN_AMD_FP32_MODE", "exact")
+if _fp32_mode not in ("exact", "fast"):
+    raise ValueError(f"HBSATTN_AMD_FP32_MODE must be 'exact' or 'fast', not {_fp32_mode!r}")
+
+
+def set_fp32_mode(mode: str) -> str:
+    """Selects how fp32 inputs are multiplied ("exact" or "fast"); returns the previous mode."""
+    global _fp32_mode
+    if mode not in ("exact", "fast"):
+        raise ValueError(f"fp32 mode must be 'exact' or 'fast', not {mode!r}")
+    previous, _fp32_mode = _fp32_mode, mode
+    return previous
+
+
+def _dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32 and _fp32_mode == "fast":
+        return _lib.DTYPE_F32_STAGED16
+    return _DTYPE_CODES[dtype]
 
 
 def _as_int32(t: torch.Tensor) -> torch.Tensor:
@@ -74,8 +98,8 @@ def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_s
     ws_bytes = int(lib.hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block))
     if staging is not None:
         total_q, total_k, nhead_q, headdim = staging
-        ws_bytes = int(lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F32, total_q, total_k, nhead_q, nhead_k, headdim,
-                                                          num_q_block, num_k_block))
+        ws_bytes = int(lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F32_STAGED16, total_q, total_k, nhead_q, nhead_k,
+                                                          headdim, num_q_block, num_k_block))
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     cu_q, cu_k = _as_int32(cu_q_seqlens), _as_int32(cu_k_seqlens)
     qb2b, cu_nqb, cu_nkb = _as_int32(q_block_to_batch), _as_int32(cu_num_q_block), _as_int32(cu_num_k_block)
@@ -132,8 +156,9 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = 
     strides = (ctypes.c_int64 * 8)(q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
                                    out_run.stride(0), out_run.stride(1))
     ws = prepared.workspace
-    if q.dtype == torch.float32:   # room for the fp16 staging copies behind the work description
-        need = int(lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F32, total_q, total_k, nhead_q, nhead_k, d_run,
+    code = _dtype_code(q.dtype)
+    if code == _lib.DTYPE_F32_STAGED16:   # room for the fp16 staging copies behind the work description
+        need = int(lib.hbsa_fwd_workspace_bytes_dtype(code, total_q, total_k, nhead_q, nhead_k, d_run,
                                                       prepared.num_q_block, prepared.num_k_block))
         if ws.numel() < need:
             grown = torch.empty(need, dtype=torch.uint8, device=ws.device)
@@ -143,7 +168,7 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = 
         lse_strides = (ctypes.c_int64 * 2)(*lse.stride()) if return_lse else None
         rc = lib.hbsa_fwd_run_lse(q.data_ptr(), k.data_ptr(), v.data_ptr(), out_run.data_ptr(),
                                   lse.data_ptr() if return_lse else None, lse_strides, ws.data_ptr(), ws.numel(),
-                                  _DTYPE_CODES[q.dtype], total_q, total_k, nhead_q, nhead_k, d_run, prepared.num_q_block,
+                                  code, total_q, total_k, nhead_q, nhead_k, d_run, prepared.num_q_block,
                                   prepared.num_k_block, prepared.q_block_size, prepared.k_block_size,
                                   int(prepared.causal), scale, strides, torch.cuda.current_stream().cuda_stream)
     if rc != 0:
@@ -165,7 +190,7 @@ def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, 
         raise RuntimeError("q, k, v and block_mask must live on the same device")
     assert q.shape[1] % k.shape[1] == 0, "nhead_q must be divisible by nhead_k (for GQA)"
     staging = None
-    if q.dtype == torch.float32 and q.dim() == 3 and k.dim() == 3:
+    if q.dtype == torch.float32 and _fp32_mode == "fast" and q.dim() == 3 and k.dim() == 3:
         staging = (q.shape[0], k.shape[0], q.shape[1], next((d for d in _NATIVE_HEADDIMS if d >= q.shape[2]), q.shape[2]))
     prepared = hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, num_q_block,
                             q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, staging)

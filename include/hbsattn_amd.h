@@ -35,7 +35,8 @@ extern "C" {
  * hbsattn/fwd_triton_auto_tile_size.py:272) */
 #define HBSA_DTYPE_BF16 0
 #define HBSA_DTYPE_F16 1
-#define HBSA_DTYPE_F32 2 /* see hbsa_fwd_workspace_bytes_dtype */
+#define HBSA_DTYPE_F32 2          /* fp32 tensors, fp32 matrix instructions: the reference's fp32 arithmetic */
+#define HBSA_DTYPE_F32_STAGED16 3 /* fp32 tensors, 16-bit matrix instructions: see hbsa_fwd_workspace_bytes_dtype */
 
 #define HBSA_ERR_INVALID_ARGUMENT (-1)
 #define HBSA_ERR_UNSUPPORTED (-2)
@@ -70,17 +71,20 @@ int hbsa_calculate_blocks(const int32_t *cu_seqlen, int32_t batch, int32_t block
 size_t hbsa_fwd_workspace_bytes(int32_t nhead_k, int32_t num_q_block, int32_t num_k_block);
 
 /*
- * The same for a given element type.  For HBSA_DTYPE_BF16 / HBSA_DTYPE_F16 it equals
- * hbsa_fwd_workspace_bytes.  For HBSA_DTYPE_F32 (the reference accepts fp32 q/k/v, its tests use
- * them: reference test/test_accuracy.py:24) it adds room for fp16 staging copies of q, k and v:
- * fp32 tensors are multiplied by a power of two chosen from their largest magnitude (found on the
- * device, no host synchronisation) and rounded to fp16, the products accumulate in fp32, the
- * softmax runs in fp32 and `out` is written as fp32.  Operands therefore carry 11-bit
- * significands (fp32's range is kept by the scaling): on unit-scale data the result differs
- * from an all-fp32 evaluation by about 1e-3 at most, inside the reference's own test tolerance
- * (allclose with atol = rtol = 1e-2, reference test/test_accuracy.py:87-89) but coarser than the
- * reference's fp32 dot products (tl.dot(..., allow_tf32=False),
- * reference hbsattn/fwd_triton_auto_tile_size.py:205,225).
+ * The same for a given element type.  For every type but HBSA_DTYPE_F32_STAGED16 it equals
+ * hbsa_fwd_workspace_bytes.
+ *
+ * fp32 q/k/v/out (the reference accepts them, its tests use them: reference
+ * test/test_accuracy.py:24) come in two forms.  HBSA_DTYPE_F32 multiplies fp32 operands with fp32
+ * matrix instructions, as the reference's fp32 path does (tl.dot(..., allow_tf32=False), reference
+ * hbsattn/fwd_triton_auto_tile_size.py:205,225), at the fp32 matrix rate, a sixteenth of the bf16
+ * one.  HBSA_DTYPE_F32_STAGED16 is the fast form: each tensor is multiplied by a power of two
+ * chosen from its largest magnitude (found on the device, no host synchronisation) and rounded to
+ * fp16 staging copies in the workspace, the 16-bit kernel runs on those with fp32 accumulation and
+ * softmax, and `out` is written as fp32.  Its operands carry 11-bit significands (fp32's range is
+ * kept by the scaling): on unit-scale data the result differs from an all-fp32 evaluation by about
+ * 1e-3 at most, inside the reference's own test tolerance (allclose with atol = rtol = 1e-2,
+ * reference test/test_accuracy.py:87-89).
  * hbsa_fwd_prepare needs only the hbsa_fwd_workspace_bytes prefix.
  */
 size_t hbsa_fwd_workspace_bytes_dtype(int32_t dtype, int32_t total_q, int32_t total_k,

@@ -8,10 +8,13 @@ from oracle.dense import hbsa_oracle
 # North-star tolerance for 16-bit inputs against the fp32 masked-dense oracle.
 MAX_ABS_TOL = 2e-2
 MEAN_ABS_TOL = 2e-3
-# fp32 inputs are computed with 11-bit significands for q, k, v and p (fp32 accumulation and softmax),
-# like the reference's tf32 dot products: an order of magnitude tighter than the 16-bit bar.
+# fp32 inputs, "fast" mode: 11-bit significands for q, k, v and p (fp32 accumulation and softmax).
 F32_MAX_ABS_TOL = 4e-3
 F32_MEAN_ABS_TOL = 3e-4
+# fp32 inputs, "exact" mode: fp32 operands and matrix instructions, against the fp32 torch oracle
+# (both sum in fp32, in different orders)
+F32_EXACT_MAX_ABS_TOL = 2e-5
+F32_EXACT_MEAN_ABS_TOL = 2e-6
 
 
 def oracle_for(w, **kw) -> torch.Tensor:
@@ -23,8 +26,14 @@ def oracle_for(w, **kw) -> torch.Tensor:
 def assert_close_to_oracle(out: torch.Tensor, ref: torch.Tensor, what: str = "", max_abs: float = None,
                            mean_abs: float = None) -> None:
     f32 = out.dtype == torch.float32
-    max_abs = max_abs if max_abs is not None else (F32_MAX_ABS_TOL if f32 else MAX_ABS_TOL)
-    mean_abs = mean_abs if mean_abs is not None else (F32_MEAN_ABS_TOL if f32 else MEAN_ABS_TOL)
+    if f32:
+        from hbsattn_amd import interface
+        exact = interface._fp32_mode == "exact"
+        dflt = (F32_EXACT_MAX_ABS_TOL, F32_EXACT_MEAN_ABS_TOL) if exact else (F32_MAX_ABS_TOL, F32_MEAN_ABS_TOL)
+    else:
+        dflt = (MAX_ABS_TOL, MEAN_ABS_TOL)
+    max_abs = max_abs if max_abs is not None else dflt[0]
+    mean_abs = mean_abs if mean_abs is not None else dflt[1]
     out = out.detach().float().cpu()
     sel = ~torch.isnan(ref)
     assert sel.any(), "oracle computed nothing"

@@ -53,7 +53,8 @@ def test_workspace_bytes_per_dtype():
     args = (1000, 2000, 32, 8, 128, 64, 64)
     assert lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_BF16, *args) == base
     assert lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F16, *args) == base
-    f32 = lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F32, *args)
+    assert lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F32, *args) == base   # fp32 matrix instructions: no staging
+    f32 = lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F32_STAGED16, *args)
     staged = (1000 * 32 + 2 * 2000 * 8) * 128 * 2          # fp16 copies of q, k and v
     assert base + staged <= f32 <= base + staged + 3 * 256 and f32 % 256 == 0
 
