@@ -410,3 +410,34 @@ def test_very_long_key_sequences_refill_the_tile_list(kbs, keep, causal):
     out = _run(w)
     assert_close_to_oracle(out, oracle_for(w), f"long keys kbs={kbs}")
     assert torch.equal(out, _run(w))
+
+
+# ---------------------------------------------------------------------------------------
+# graph capture: the launches of a call are plain kernels on the caller's stream
+# ---------------------------------------------------------------------------------------
+def test_call_can_be_captured_in_a_graph_and_replayed():
+    w = make_problem(seed=61, q_lens=[1024, 300], k_lens=[1024, 700], hq=8, hk=4, d=128, qbs=128, kbs=128, keep=0.5,
+                     diag=True, causal=True, scale=None)
+    args = list(w.args())
+    eager0 = HBSAttention(*args).clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        HBSAttention(*args)                                   # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = HBSAttention(*args)
+    for step in range(4):                                     # every replay is checked, with eager work in between
+        if step:
+            w.q.copy_(torch.randn_like(w.q))                  # new inputs in place: the graph reads the same buffers
+            w.v.mul_(-0.5)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = HBSAttention(*args)
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager), f"replay {step}"
+        if step == 0:
+            assert torch.equal(captured, eager0)
