@@ -55,6 +55,7 @@ constexpr int kThreads = 256;   // 4 wavefronts
 constexpr int kWaveRows = 32;   // query rows per wavefront (the MFMA N dimension)
 constexpr int kTileKeys = 64;   // keys per main-loop step
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kMaxDevices = 64;            // devices of one process the launch caches cover
 constexpr float kLazyRescaleLog2 = 8.0f;  // running max may lag the true max by 2^8
 
 // Geometry of one q block, written by the pre-pass (32 bytes).
@@ -1095,7 +1096,12 @@ template <int D, typename E, bool OUT32>
 int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
   constexpr int lds_bytes = 4 * kTileKeys * D * 2 + 2 * H_WORDS * 4 + 2 * kListCap * 4;
   const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E, OUT32>);
-  static thread_local int resident = 0;   // workgroups that fit the device at once
+  // workgroups that fit the current device at once; the attribute and the occupancy are per device
+  static thread_local int resident_of[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(HBSA_ERR_UNSUPPORTED, "no current device, or device index above %d", kMaxDevices - 1);
+  int &resident = resident_of[dev];
   if (resident == 0) {
     hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
@@ -1268,11 +1274,14 @@ template <int D>
 int launch_fwd_f32(const FwdParams &fp, float c_signed, long long items, hipStream_t stream) {
   constexpr int lds_bytes = 2 * kTileKeys * (D + 4) * 4;
   const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_f32_kernel<D>);
-  static thread_local bool configured = false;
-  if (!configured) {
+  static thread_local bool configured[kMaxDevices] = {};   // the attribute is per device
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(HBSA_ERR_UNSUPPORTED, "no current device, or device index above %d", kMaxDevices - 1);
+  if (!configured[dev]) {
     hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
+    configured[dev] = true;
   }
   hipLaunchKernelGGL((hbsa_fwd_f32_kernel<D>), dim3((unsigned)items), dim3(kThreads), lds_bytes, stream, fp, c_signed);
   hipError_t e = hipGetLastError();
