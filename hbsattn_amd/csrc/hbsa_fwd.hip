@@ -598,13 +598,15 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   auto tile_ptr = [&](const char *base, int tok, uint32_t stride) {   // tok >= 0
     return base + (uint64_t)(uint32_t)tok * (uint64_t)stride;
   };
-  auto issue_loads = [&](int buf, const char *kbase, const char *vbase, int valid) {
+  // One operand's half of a tile's loads.  V_PART selects the V buffers (which follow the K buffers).
+  auto issue_part = [&](auto v_part_, int buf, const char *base, int valid) {
+    constexpr bool V_PART = decltype(v_part_)::value;
+    constexpr int lds_off = V_PART ? 2 * TILE_BYTES : 0;
     const uint32_t l0 = lds_k_addr + (uint32_t)(buf * TILE_BYTES) + (uint32_t)wave * 1024u;
     if (valid == kTileKeys) {
       static_for<0, LOADS>([&](auto i_) {
         constexpr int i = decltype(i_)::value;
-        dma16(std::integral_constant<int, i * 4096>{}, kbase, ld_koff[i], l0);
-        dma16(std::integral_constant<int, 2 * TILE_BYTES + i * 4096>{}, vbase, ld_voff[i], l0);
+        dma16(std::integral_constant<int, lds_off + i * 4096>{}, base, V_PART ? ld_voff[i] : ld_koff[i], l0);
       });
     } else {   // ragged tail of a run: rows past the end re-read the last valid row (masked later)
       static_for<0, LOADS>([&](auto i_) {
@@ -612,10 +614,15 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         int r; uint32_t kc, vc;
         ld_place(i, r, kc, vc);
         r = min(r, valid - 1);
-        dma16(std::integral_constant<int, i * 4096>{}, kbase, (uint32_t)r * ks32 + kc, l0);
-        dma16(std::integral_constant<int, 2 * TILE_BYTES + i * 4096>{}, vbase, (uint32_t)r * vs32 + vc, l0);
+        dma16(std::integral_constant<int, lds_off + i * 4096>{}, base, (uint32_t)r * (V_PART ? vs32 : ks32) + (V_PART ? vc : kc), l0);
       });
     }
+  };
+  auto issue_k = [&](int buf, const char *kbase, int valid) { issue_part(std::false_type{}, buf, kbase, valid); };
+  auto issue_v = [&](int buf, const char *vbase, int valid) { issue_part(std::true_type{}, buf, vbase, valid); };
+  auto issue_loads = [&](int buf, const char *kbase, const char *vbase, int valid) {
+    issue_k(buf, kbase, valid);
+    issue_v(buf, vbase, valid);
   };
 
   // per-lane LDS read addresses
@@ -743,6 +750,8 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         __syncthreads();                     // ... for every wave, and the other buffers are free
 
         const bool last = chunk_base + t + 1 == total;
+        int nx_valid = 0;                 // > 0: a next tile exists and its loads go out during this tile
+        const char *nx_vbase = nullptr;
         if (t + 1 < n) {
           int e1;
           if (((t + 1) & 63) == 0) {
@@ -752,18 +761,24 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
             e1 = __builtin_amdgcn_readlane(held, (t + 1) & 63);
           }
           const int tok = (e1 >> 6) << 4;
-          issue_loads(buf ^ 1, tile_ptr(kg, tok, ks32), tile_ptr(vg, tok, vs32), (e1 & 63) + 1);
+          nx_valid = (e1 & 63) + 1;
+          nx_vbase = tile_ptr(vg, tok, vs32);
+          issue_k(buf ^ 1, tile_ptr(kg, tok, ks32), nx_valid);
         } else if (last) {
           nxt_hk = hdr_word(c ^ 1, H_HK);
           if (nxt_hk >= 0 && hdr_word(c ^ 1, H_TOTAL) > 0) {
             const int e1 = __builtin_amdgcn_readfirstlane(lds_list[(c ^ 1) * kListCap]);
             const int tok = hdr_word(c ^ 1, H_KEY_BEGIN) + ((e1 >> 6) << 4);
-            issue_loads(buf ^ 1, tile_ptr(p.k + (int64_t)nxt_hk * p.k_h, tok, ks32),
-                        tile_ptr(p.v + (int64_t)nxt_hk * p.v_h, tok, vs32), (e1 & 63) + 1);
+            nx_valid = (e1 & 63) + 1;
+            nx_vbase = tile_ptr(p.v + (int64_t)nxt_hk * p.v_h, tok, vs32);
+            issue_k(buf ^ 1, tile_ptr(p.k + (int64_t)nxt_hk * p.k_h, tok, ks32), nx_valid);
           }
         }
+        // The next tile's K is requested above, its V only after the first MFMA block below: the
+        // four wavefronts then do not all queue at the load unit at once, and V is needed later.
 
         const bool compute = active && (!p.causal || kpos <= wave_kvis_max);
+        if (!compute && nx_valid > 0) issue_v(buf ^ 1, nx_vbase, nx_valid);
         if (compute) {
           // The tile is processed as two halves of 32 keys so that, inside one wavefront, the
           // matrix cores always have work queued while the vector ALU does the softmax of the
@@ -797,6 +812,8 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
             s0 = E::mfma(kb[i % PF], qf[i % KSTEPS], s0);
             if constexpr (i + PF < NK) read_k(std::integral_constant<int, i + PF>{});
           });
+
+          if (nx_valid > 0) issue_v(buf ^ 1, nx_vbase, nx_valid);
 
           // row max of one half, merged into the running max; O and l are rescaled (rarely:
           // the running max may lag the true one by 2^kLazyRescaleLog2)
