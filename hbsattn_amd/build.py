@@ -6,6 +6,7 @@ cross-compiles, so no GPU is needed to build.
 from __future__ import annotations
 
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -23,13 +24,34 @@ HIPCC_FLAGS = [
 ]
 
 
+def _vgpr_spills(remarks: str) -> dict:
+    """Kernels with vector-register spills, from the compiler's resource-usage remarks."""
+    spills, name = {}, None
+    for line in remarks.splitlines():
+        m = re.search(r"remark:\s+Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.search(r"remark:\s+VGPRs Spill: (\d+)", line)
+        if m and name is not None and int(m.group(1)) > 0:
+            spills[name] = int(m.group(1))
+    return spills
+
+
 def build(verbose: bool = False) -> str:
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    cmd = [hipcc] + HIPCC_FLAGS + SOURCES + ["-o", OUTPUT]
+    cmd = [hipcc] + HIPCC_FLAGS + ["-Rpass-analysis=kernel-resource-usage"] + SOURCES + ["-o", OUTPUT]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
         raise RuntimeError("hipcc failed: " + " ".join(cmd))
+    # The attention kernels issue their LDS reads by hand and wait for them by count.  The compiler
+    # does not know that such a register has a read in flight; if it spills one, it saves the
+    # register before the data has arrived and the result is wrong now and then.  So a build in
+    # which any kernel spills vector registers is refused.
+    spills = _vgpr_spills(res.stderr)
+    if spills:
+        os.remove(OUTPUT)
+        raise RuntimeError(f"vector-register spills in {spills}: reduce register pressure (see the comment here)")
     if verbose:
         print(" ".join(cmd))
     return OUTPUT
