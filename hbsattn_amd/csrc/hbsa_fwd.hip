@@ -751,7 +751,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 
         const bool last = chunk_base + t + 1 == total;
         int nx_valid = 0;                 // > 0: a next tile exists and its loads go out during this tile
-        const char *nx_vbase = nullptr;
+        const char *nx_vbase = nullptr, *nx_kbase = nullptr;
         if (t + 1 < n) {
           int e1;
           if (((t + 1) & 63) == 0) {
@@ -763,7 +763,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
           const int tok = (e1 >> 6) << 4;
           nx_valid = (e1 & 63) + 1;
           nx_vbase = tile_ptr(vg, tok, vs32);
-          issue_k(buf ^ 1, tile_ptr(kg, tok, ks32), nx_valid);
+          nx_kbase = tile_ptr(kg, tok, ks32);
         } else if (last) {
           nxt_hk = hdr_word(c ^ 1, H_HK);
           if (nxt_hk >= 0 && hdr_word(c ^ 1, H_TOTAL) > 0) {
@@ -771,14 +771,17 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
             const int tok = hdr_word(c ^ 1, H_KEY_BEGIN) + ((e1 >> 6) << 4);
             nx_valid = (e1 & 63) + 1;
             nx_vbase = tile_ptr(p.v + (int64_t)nxt_hk * p.v_h, tok, vs32);
-            issue_k(buf ^ 1, tile_ptr(p.k + (int64_t)nxt_hk * p.k_h, tok, ks32), nx_valid);
+            nx_kbase = tile_ptr(p.k + (int64_t)nxt_hk * p.k_h, tok, ks32);
           }
         }
-        // The next tile's K is requested above, its V only after the first MFMA block below: the
-        // four wavefronts then do not all queue at the load unit at once, and V is needed later.
+        // The next tile's K is requested right after this tile's first operand reads, its V only after
+        // the first MFMA block: the four wavefronts then do not all queue at the load unit at once.
 
         const bool compute = active && (!p.causal || kpos <= wave_kvis_max);
-        if (!compute && nx_valid > 0) issue_v(buf ^ 1, nx_vbase, nx_valid);
+        if (!compute && nx_valid > 0) {
+          issue_k(buf ^ 1, nx_kbase, nx_valid);
+          issue_v(buf ^ 1, nx_vbase, nx_valid);
+        }
         if (compute) {
           // The tile is processed as two halves of 32 keys so that, inside one wavefront, the
           // matrix cores always have work queued while the vector ALU does the softmax of the
@@ -804,6 +807,8 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
             else kb[i % PF] = lds_read_b128<32 * RB>(k_addr[ks]);
           };
           static_for<0, PF>(read_k);
+          // the next tile's K is requested while this tile's first operands are on their way from LDS
+          if (nx_valid > 0) issue_k(buf ^ 1, nx_kbase, nx_valid);
           // ---- S0 = K[0:32] . Q^T
           static_for<0, KSTEPS>([&](auto i_) {
             constexpr int i = decltype(i_)::value;
