@@ -441,3 +441,40 @@ def test_call_can_be_captured_in_a_graph_and_replayed():
         assert torch.equal(captured, eager), f"replay {step}"
         if step == 0:
             assert torch.equal(captured, eager0)
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_fp16_medium_problem(d):
+    w = make_problem(seed=71, q_lens=[1500, 640], k_lens=[1500, 2048], hq=8, hk=4, d=d, qbs=128, kbs=64, keep=0.35, diag=True,
+                     causal=True, scale=None, dtype=torch.float16)
+    out = _run(w)
+    assert out.dtype == torch.float16
+    assert_close_to_oracle(out, oracle_for(w), f"fp16 d={d}")
+    assert torch.equal(out, _run(w))
+
+
+def test_strided_output_through_the_c_entry_point():
+    # `out` with padding between heads and tokens: the library writes only the rows' own 16-byte chunks
+    import ctypes
+    from hbsattn_amd import _lib
+    w = make_problem(seed=72, q_lens=[300, 77], k_lens=[300, 200], hq=4, hk=2, d=64, qbs=64, kbs=64, keep=0.5, diag=True,
+                     causal=True, scale=None)
+    lib = _lib.load()
+    nqb, _, qb2b, cu_nqb = w.q_meta
+    nkb, _, _, cu_nkb = w.k_meta
+    i32 = lambda t: t.to(torch.int32).contiguous()
+    cu_q, cu_k, qb2b, cu_nqb, cu_nkb = map(i32, (w.cu_q_seqlens, w.cu_k_seqlens, qb2b, cu_nqb, cu_nkb))
+    wide = torch.full((w.q.shape[0], 4, 96), 7.0, dtype=torch.bfloat16, device="cuda")
+    out = wide[:, :, 16:80]
+    need = lib.hbsa_fwd_workspace_bytes(2, nqb, nkb)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    strides = (ctypes.c_int64 * 11)(w.q.stride(0), w.q.stride(1), w.k.stride(0), w.k.stride(1), w.v.stride(0), w.v.stride(1),
+                                    out.stride(0), out.stride(1), *w.block_mask.stride())
+    rc = lib.hbsa_fwd(w.q.data_ptr(), w.k.data_ptr(), w.v.data_ptr(), out.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),
+                      w.block_mask.data_ptr(), qb2b.data_ptr(), cu_nqb.data_ptr(), cu_nkb.data_ptr(), ws.data_ptr(), need, 0,
+                      2, w.q.shape[0], w.k.shape[0], 4, 2, 64, nqb, nkb, 64, 64, 1, 64 ** -0.5, strides,
+                      torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0, _lib.last_error()
+    assert torch.equal(out, _run(w))
+    assert (wide[:, :, :16] == 7).all() and (wide[:, :, 80:] == 7).all()
