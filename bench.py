@@ -128,8 +128,9 @@ def measure(name, steps, warmup):
 
 
 def cpu_baseline(w, budget_s=20.0):
-    """The CPU oracle on sequence 0 of the workload, one kv head group at a time until the
-    budget is spent; throughput in the metric's unit from the sample's own visited blocks."""
+    """The CPU oracle on (sequence, kv head) pairs of the workload, in sequence-major order, one
+    pair at a time until the budget is spent; throughput in the metric's unit from the sample's own
+    visited blocks."""
     from hbsattn_amd.workloads import Workload, count_work
     from oracle.dense import hbsa_oracle
 
