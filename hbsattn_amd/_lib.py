@@ -52,6 +52,8 @@ def load() -> ctypes.CDLL:
     lib.hbsa_fwd_run_lse.restype = ctypes.c_int
     lib.hbsa_fwd_run_lse.argtypes = ([vp] * 5 + [i64p, vp, ctypes.c_size_t] + [ctypes.c_int32] * 11
                                      + [ctypes.c_float, i64p, vp])
+    lib.hbsa_fwd_split_workspace_bytes.restype = ctypes.c_size_t
+    lib.hbsa_fwd_split_workspace_bytes.argtypes = [ctypes.c_int32] * 7
     lib.hbsa_calculate_blocks.restype = ctypes.c_int
     lib.hbsa_calculate_blocks.argtypes = [vp, ctypes.c_int32, ctypes.c_int32, vp, vp, vp, vp, ctypes.c_int32]
     _lib = lib

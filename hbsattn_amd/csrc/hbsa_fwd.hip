@@ -114,6 +114,14 @@ struct FwdParams {
   struct Sched *sched;
   float *lse;             // optional [total_q, nhead_q] log-sum-exp output (nullptr: none)
   int64_t lse_s, lse_h;   // its strides in elements
+  // Split over key blocks (few, long work items): every (kv head, q block, slot group) becomes
+  // nparts items, part i sees the bit row copy i (its share of the k blocks) and stores a
+  // normalised fp32 partial result and its log-sum-exp; hbsa_merge_kernel combines them.
+  int32_t nparts;         // 1: no split
+  FastDiv div_nparts;
+  float *part_out;        // [nparts, total_q, nhead_q, D]
+  float *part_lse;        // [nparts, total_q, nhead_q]
+  int32_t total_q, nhead_q;
 };
 
 // --------------------------------------------------------------------------------------
@@ -322,7 +330,7 @@ __global__ __launch_bounds__(256) void hbsa_f32_stage_kernel(F32Tensor t, const 
 constexpr int kListCap = 1024;   // tile entries per list; longer items are expanded in chunks
 
 // Item header in LDS (16 ints).
-enum { H_HK = 0, H_QB, H_SUB, H_TOTAL, H_ROW_BEGIN, H_ROWS, H_KEY_BEGIN, H_Q_POS, H_SHIFT, H_WORDS = 16 };
+enum { H_HK = 0, H_QB, H_SUB, H_TOTAL, H_ROW_BEGIN, H_ROWS, H_KEY_BEGIN, H_Q_POS, H_SHIFT, H_PART, H_WORDS = 16 };
 
 __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
@@ -495,12 +503,12 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   const int first_queue = home < nq ? home : home % nq;
   int tries = 0;                    // queues found empty so far
   uint32_t pending = 0xffffffffu;   // queue index claimed for the item after the staged one
-  int st_hk = -1, st_qb = 0, st_sub = 0;   // staged item: claimed, records fetched, list not built
+  int st_hk = -1, st_qb = 0, st_sub = 0, st_part = 0;   // staged item: claimed, records fetched, list not built
   uint32_t st_info = 0, st_bits = 0;       // lane i: word i of its QBlockInfo / of its bit row
 
   auto queue_len = [&](int v) -> uint32_t {
     const int heads = v < p.nhead_k ? (p.nhead_k - v + 7) / 8 : 0;
-    return (uint32_t)heads * (uint32_t)p.nqb * (uint32_t)p.nsub;
+    return (uint32_t)heads * (uint32_t)p.nqb * (uint32_t)p.nsub * (uint32_t)p.nparts;
   };
   auto claim = [&]() -> uint32_t {   // the value is looked at an item later, so its latency is hidden
     uint32_t r = 0xffffffffu;
@@ -517,8 +525,10 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     while (tries < 8) {
       const int v = (first_queue + tries) & 7;
       if (claimed < queue_len(v)) {
-        const uint32_t t = fast_div(claimed, p.div_nsub);
-        st_sub = (int)(claimed - t * (uint32_t)p.nsub);
+        const uint32_t whole = fast_div(claimed, p.div_nparts);   // parts of one item are neighbours in the queue
+        st_part = (int)(claimed - whole * (uint32_t)p.nparts);
+        const uint32_t t = fast_div(whole, p.div_nsub);
+        st_sub = (int)(whole - t * (uint32_t)p.nsub);
         const uint32_t hq8 = fast_div(t, p.div_nqb);
         st_hk = v + 8 * (int)hq8;
         st_qb = p.nqb - 1 - (int)(t - hq8 * (uint32_t)p.nqb);
@@ -533,7 +543,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     }
     if (st_hk >= 0) {
       st_info = lane < 8 ? ((const uint32_t *)(p.info + st_qb))[lane] : 0u;
-      st_bits = lane < p.wpr ? p.bits[((size_t)st_hk * p.nqb + st_qb) * p.wpr + lane] : 0u;
+      st_bits = lane < p.wpr ? p.bits[(((size_t)st_part * p.nhead_k + st_hk) * p.nqb + st_qb) * p.wpr + lane] : 0u;
     }
   };
   // expand the staged item into list `c` and write its header
@@ -543,11 +553,12 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     if (st_hk >= 0) {
       const int nkblk = __builtin_amdgcn_readlane((int)st_info, 6);
       const int kmax = __builtin_amdgcn_readlane((int)st_info, 7);
-      total = build_tile_list(lds_list + c * kListCap, 0, p.bits + ((size_t)st_hk * p.nqb + st_qb) * p.wpr,
+      total = build_tile_list(lds_list + c * kListCap, 0,
+                              p.bits + (((size_t)st_part * p.nhead_k + st_hk) * p.nqb + st_qb) * p.wpr,
                               2 * ((nkblk + 63) >> 6), p.kbs, p.div_kbs, kmax, st_bits, lane);
     }
     if (lane == 0) {
-      hdr[H_HK] = st_hk; hdr[H_QB] = st_qb; hdr[H_SUB] = st_sub; hdr[H_TOTAL] = total;
+      hdr[H_HK] = st_hk; hdr[H_QB] = st_qb; hdr[H_SUB] = st_sub; hdr[H_TOTAL] = total; hdr[H_PART] = st_part;
     }
     if (lane < 8) {   // QBlockInfo words: row_begin, rows, key_begin, klen, q_pos, shift, nkblk, kmax
       const int dst = lane == 0 ? H_ROW_BEGIN : lane == 1 ? H_ROWS : lane == 2 ? H_KEY_BEGIN : lane == 4 ? H_Q_POS
@@ -702,6 +713,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   for (;;) {   // ------------------------------------------------------ one iteration per work item
     const int cur_hk = hdr_word(c, H_HK);
     const int cur_sub = hdr_word(c, H_SUB);
+    const int cur_part = hdr_word(c, H_PART);   // read now: wavefront 0 rewrites the header while others finish this item
     const int total = hdr_word(c, H_TOTAL);
     const int row_begin = hdr_word(c, H_ROW_BEGIN);
     const int rows = hdr_word(c, H_ROWS);
@@ -981,7 +993,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         // (the staged records now belong to a later item, so this item's are fetched again)
         const int qb = hdr_word(c, H_QB);
         const QBlockInfo inf = p.info[qb];
-        const uint32_t *row = p.bits + ((size_t)cur_hk * p.nqb + qb) * p.wpr;
+        const uint32_t *row = p.bits + (((size_t)cur_part * p.nhead_k + cur_hk) * p.nqb + qb) * p.wpr;
         const int nwords = 2 * ((inf.nkblk + 63) >> 6);
         (void)build_tile_list(lds_list + c * kListCap, chunk_base, row, nwords, p.kbs, p.div_kbs, inf.kmax,
                               lane < nwords ? row[lane] : 0u, lane);
@@ -998,6 +1010,22 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     if (active) {
       const float l_tot = half_sum(l_run);
       const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;   // 1 ulp; a full division is ten instructions
+      if (p.nparts > 1) {
+        // split over key blocks: this part's normalised result and log-sum-exp, for the merge kernel
+        if (l32 < nrows) {
+          const int64_t rh = ((int64_t)cur_part * p.total_q + (row_begin + row0 + l32)) * p.nhead_q + hq;
+          if (g32 == 0)
+            p.part_lse[rh] = l_tot > 0.f ? (m_run * sm_c + __builtin_amdgcn_logf(l_tot)) * 0.69314718055994531f : -INFINITY;
+          float *dst = p.part_out + rh * D;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+              f32x4 w = {o[dt][4 * i4 + 0] * inv, o[dt][4 * i4 + 1] * inv, o[dt][4 * i4 + 2] * inv, o[dt][4 * i4 + 3] * inv};
+              *(f32x4 *)(dst + dt * 32 + 8 * i4 + 4 * g32) = w;
+            }
+        }
+      } else {
       if (p.lse != nullptr && g32 == 0 && l32 < nrows) {
         // natural-log sum over the row's visible keys of exp(scale * q.k); m_run is the (possibly
         // lagging) reference maximum the row sum was accumulated under, which makes this exact
@@ -1026,6 +1054,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
               *(u32x2 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 2) = w;
             }
         }
+      }
       }
     }
 
@@ -1058,6 +1087,65 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     }
     if (nxt_hk < 0) break;
     c ^= 1;
+  }
+}
+
+// Split over key blocks: bit row copy `part` keeps the k blocks [part * n / nparts, (part + 1) * n / nparts)
+// of a q block's own sequence (n = its k blocks).
+__global__ __launch_bounds__(256) void hbsa_split_bits_kernel(const uint32_t *bits, uint32_t *out, const QBlockInfo *info,
+                                                              int nhead_k, int nqb, int wpr, int nparts) {
+  const int64_t per_part = (int64_t)nhead_k * nqb * wpr;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= per_part * nparts) return;
+  const int part = (int)(i / per_part);
+  const int64_t r = i % per_part;
+  const int w = (int)(r % wpr), qb = (int)((r / wpr) % nqb);
+  const int n = info[qb].nkblk;
+  const int lo = (int)((int64_t)part * n / nparts), hi = (int)((int64_t)(part + 1) * n / nparts);
+  uint32_t m = 0;
+  for (int b = 0; b < 32; ++b) {
+    const int j = w * 32 + b;
+    if (j >= lo && j < hi) m |= 1u << b;
+  }
+  out[i] = bits[r] & m;
+}
+
+// out[row, head, :] = sum over parts of exp(lse_part - lse) * partial, lse = log sum exp(lse_part);
+// rows whose parts all saw no key give 0 (and lse -inf).  One thread per 4 output elements.
+template <typename E, bool OUT32>
+__global__ __launch_bounds__(256) void hbsa_merge_kernel(const float *part_out, const float *part_lse, char *out, float *lse,
+                                                         const Sched *sched, int nparts, int total_q, int nhead_q, int dshift,
+                                                         int64_t o_s, int64_t o_h, int64_t lse_s, int64_t lse_h) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t rows = (int64_t)total_q * nhead_q;
+  if (i >= rows << dshift) return;
+  const int64_t rh = i >> dshift;
+  const int dq = (int)(i & ((1 << dshift) - 1));
+  float mx = -INFINITY;
+  for (int pt = 0; pt < nparts; ++pt) mx = fmaxf(mx, part_lse[pt * rows + rh]);
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  float den = 0.f;
+  if (mx != -INFINITY) {
+    for (int pt = 0; pt < nparts; ++pt) {
+      const float l = part_lse[pt * rows + rh];
+      if (l == -INFINITY) continue;
+      const float w = __expf(l - mx);
+      den += w;
+      acc += *(const f32x4 *)(part_out + (((int64_t)pt * rows + rh) << (dshift + 2)) + dq * 4) * w;
+    }
+    acc *= 1.f / den;
+  }
+  const int64_t row = rh / nhead_q, h = rh % nhead_q;
+  if (lse != nullptr && dq == 0) lse[row * lse_s + h * lse_h] = mx == -INFINITY ? -INFINITY : mx + __logf(den);
+  char *dst = out + row * o_s + h * o_h;
+  if constexpr (OUT32) {
+    acc *= sched->out_mul;
+    *(f32x4 *)(dst + dq * 16) = acc;
+  } else {
+    u32x2 w;
+    w.x = E::pack2(acc[0], acc[1]);
+    w.y = E::pack2(acc[2], acc[3]);
+    *(u32x2 *)(dst + dq * 8) = w;
   }
 }
 
@@ -1102,6 +1190,33 @@ F32Tensor f32_tensor(int i, const void *q, const void *k, const void *v, const i
   const int64_t tokens = i == 0 ? total_q : total_k;
   const int heads = i == 0 ? nhead_q : nhead_k;
   return {(const float *)x, strides[2 * i], strides[2 * i + 1], heads, dshift, tokens * heads * headdim / 4};
+}
+
+// Split over key blocks pays when the work items cannot fill the device: fewer than one per CU.
+// Returns the number of parts (1 = no split) for the current device.
+int split_parts(long long items, int num_k_block) {
+  static thread_local int cus_of[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 1;
+  if (cus_of[dev] == 0 && hipDeviceGetAttribute(&cus_of[dev], hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+    return 1;
+  const int cus = cus_of[dev];
+  if (items <= 0 || items > cus) return 1;
+  long long parts = std::min<long long>(32, (2LL * cus) / items);
+  parts = std::min<long long>(parts, num_k_block / 8);     // a part should still have a few k blocks
+  return parts < 2 ? 1 : (int)parts;
+}
+// split area: nparts bit row copies | nparts partial outputs | nparts partial log-sum-exps, each array packed
+inline size_t split_bits_bytes(int parts, int nhead_k, int num_q_block, int num_k_block) {
+  return align_up((size_t)parts * nhead_k * num_q_block * words_per_row(num_k_block) * sizeof(uint32_t), 256);
+}
+inline size_t split_out_bytes(int parts, int total_q, int nhead_q, int headdim) {
+  return align_up((size_t)parts * total_q * nhead_q * headdim * 4, 256);
+}
+inline size_t split_bytes(int parts, int total_q, int nhead_q, int nhead_k, int headdim, int num_q_block, int num_k_block) {
+  if (parts < 2) return 0;
+  return split_bits_bytes(parts, nhead_k, num_q_block, num_k_block) + split_out_bytes(parts, total_q, nhead_q, headdim) +
+         align_up((size_t)parts * total_q * nhead_q * 4, 256);
 }
 
 int persistent_grid(const void *kernel, int lds_bytes) {
@@ -1292,6 +1407,41 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_f32_kernel(FwdParams p, 
     }
 }
 
+template <int D, typename E, bool OUT32>
+int launch_fwd_split(FwdParams &fp, long long items, hipStream_t stream, char *area, int num_k_block, int total_q,
+                     int nhead_q) {
+  const int parts = fp.nparts;
+  uint32_t *bit_copies = (uint32_t *)area;
+  char *after_bits = area + split_bits_bytes(parts, fp.nhead_k, fp.nqb, num_k_block);
+  fp.part_out = (float *)after_bits;
+  fp.part_lse = (float *)(after_bits + split_out_bytes(parts, total_q, nhead_q, D));
+  {
+    const int64_t n = (int64_t)fp.nhead_k * fp.nqb * fp.wpr * parts;
+    hipLaunchKernelGGL(hbsa_split_bits_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, fp.bits,
+                       bit_copies, fp.info, fp.nhead_k, fp.nqb, fp.wpr, parts);
+  }
+  char *final_out = fp.out;
+  float *final_lse = fp.lse;
+  const int64_t o_s = fp.o_s, o_h = fp.o_h, lse_s = fp.lse_s, lse_h = fp.lse_h;
+  const size_t rows = (size_t)total_q * nhead_q;
+  fp.bits = bit_copies;
+  int rc = launch_fwd<D, E, OUT32>(fp, items * parts, stream);
+  if (rc != 0) return rc;
+  constexpr int dshift = D == 32 ? 3 : D == 64 ? 4 : 5;
+  const int64_t n = (int64_t)rows << dshift;
+  hipLaunchKernelGGL((hbsa_merge_kernel<E, OUT32>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, fp.part_out,
+                     fp.part_lse, final_out, final_lse, fp.sched, parts, total_q, nhead_q, dshift, o_s, o_h, lse_s, lse_h);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail((int)e, "hbsa_merge_kernel launch: %s", hipGetErrorString(e));
+  return 0;
+}
+
+template <int D, typename E, bool OUT32>
+int run_fwd(FwdParams &fp, long long items, hipStream_t stream, char *split_area, int num_k_block) {
+  if (fp.nparts > 1) return launch_fwd_split<D, E, OUT32>(fp, items, stream, split_area, num_k_block, fp.total_q, fp.nhead_q);
+  return launch_fwd<D, E, OUT32>(fp, items, stream);
+}
+
 template <int D>
 int launch_fwd_f32(const FwdParams &fp, float c_signed, long long items, hipStream_t stream) {
   constexpr int lds_bytes = 2 * kTileKeys * (D + 4) * 4;
@@ -1358,6 +1508,15 @@ size_t hbsa_fwd_workspace_bytes_dtype(int32_t dtype, int32_t total_q, int32_t to
   if (dtype == HBSA_DTYPE_F32_STAGED16 && total_q > 0 && total_k > 0 && nhead_q > 0 && nhead_k > 0 && headdim > 0)
     n += f32_stage_bytes(total_q, nhead_q, headdim) + 2 * f32_stage_bytes(total_k, nhead_k, headdim);
   return n;
+}
+
+size_t hbsa_fwd_split_workspace_bytes(int32_t total_q, int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+                                      int32_t num_q_block, int32_t num_k_block, int32_t q_block_size) {
+  if (total_q <= 0 || nhead_q <= 0 || nhead_k <= 0 || headdim <= 0 || num_q_block <= 0 || num_k_block <= 0 || q_block_size <= 0)
+    return 0;
+  const int ratio = nhead_q / nhead_k, wps = (q_block_size + kWaveRows - 1) / kWaveRows;
+  const long long items = (long long)nhead_k * num_q_block * ((ratio * wps + 3) / 4);
+  return split_bytes(split_parts(items, num_k_block), total_q, nhead_q, nhead_k, headdim, num_q_block, num_k_block);
 }
 
 int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens, const uint8_t *block_mask,
@@ -1483,6 +1642,17 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
   fp.c = c;
   const long long items = (long long)nhead_k * num_q_block * fp.nsub;
   if (items > 0x7fffffffLL) return fail(HBSA_ERR_UNSUPPORTED, "too many work items (%lld)", items);
+  // split over key blocks when the items cannot fill the device and the caller's workspace has the room
+  fp.nparts = 1;
+  fp.part_out = nullptr; fp.part_lse = nullptr;
+  fp.total_q = total_q; fp.nhead_q = nhead_q;
+  char *split_area = (char *)workspace + need;
+  if (!f32_exact) {
+    const int parts = split_parts(items, num_k_block);
+    if (parts > 1 && workspace_bytes >= need + split_bytes(parts, total_q, nhead_q, nhead_k, headdim, num_q_block, num_k_block))
+      fp.nparts = parts;
+  }
+  fp.div_nparts = make_fast_div((uint32_t)fp.nparts);
 
   if (f32_exact) {
     const float c_signed = softmax_scale * kLog2e;
@@ -1503,16 +1673,19 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
       hipLaunchKernelGGL(hbsa_f32_stage_kernel, dim3(nb), dim3(256), 0, st, t, &fp.sched->in_mul[i], (uint32_t *)dst[i]);
     }
     switch (headdim) {
-      case 32: return launch_fwd<32, ElemF16, true>(fp, items, st);
-      case 64: return launch_fwd<64, ElemF16, true>(fp, items, st);
-      default: return launch_fwd<128, ElemF16, true>(fp, items, st);
+      case 32: return run_fwd<32, ElemF16, true>(fp, items, st, split_area, num_k_block);
+      case 64: return run_fwd<64, ElemF16, true>(fp, items, st, split_area, num_k_block);
+      default: return run_fwd<128, ElemF16, true>(fp, items, st, split_area, num_k_block);
     }
   }
   const bool bf = dtype == HBSA_DTYPE_BF16;
   switch (headdim) {
-    case 32: return bf ? launch_fwd<32, ElemBF16, false>(fp, items, st) : launch_fwd<32, ElemF16, false>(fp, items, st);
-    case 64: return bf ? launch_fwd<64, ElemBF16, false>(fp, items, st) : launch_fwd<64, ElemF16, false>(fp, items, st);
-    default: return bf ? launch_fwd<128, ElemBF16, false>(fp, items, st) : launch_fwd<128, ElemF16, false>(fp, items, st);
+    case 32: return bf ? run_fwd<32, ElemBF16, false>(fp, items, st, split_area, num_k_block)
+                       : run_fwd<32, ElemF16, false>(fp, items, st, split_area, num_k_block);
+    case 64: return bf ? run_fwd<64, ElemBF16, false>(fp, items, st, split_area, num_k_block)
+                       : run_fwd<64, ElemF16, false>(fp, items, st, split_area, num_k_block);
+    default: return bf ? run_fwd<128, ElemBF16, false>(fp, items, st, split_area, num_k_block)
+                       : run_fwd<128, ElemF16, false>(fp, items, st, split_area, num_k_block);
   }
 }
 

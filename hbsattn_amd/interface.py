@@ -157,13 +157,17 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = 
                                    out_run.stride(0), out_run.stride(1))
     ws = prepared.workspace
     code = _dtype_code(q.dtype)
-    if code == _lib.DTYPE_F32_STAGED16:   # room for the fp16 staging copies behind the work description
-        need = int(lib.hbsa_fwd_workspace_bytes_dtype(code, total_q, total_k, nhead_q, nhead_k, d_run,
-                                                      prepared.num_q_block, prepared.num_k_block))
-        if ws.numel() < need:
-            grown = torch.empty(need, dtype=torch.uint8, device=ws.device)
-            grown[: ws.numel()].copy_(ws)
-            prepared.workspace = ws = grown
+    # room behind the work description for fp16 staging copies (fast fp32 mode) and for the split over
+    # key blocks the library uses when the work items cannot fill the device
+    need = int(lib.hbsa_fwd_workspace_bytes_dtype(code, total_q, total_k, nhead_q, nhead_k, d_run,
+                                                  prepared.num_q_block, prepared.num_k_block))
+    with torch.cuda.device(q.device):
+        need += int(lib.hbsa_fwd_split_workspace_bytes(total_q, nhead_q, nhead_k, d_run, prepared.num_q_block,
+                                                       prepared.num_k_block, prepared.q_block_size))
+    if ws.numel() < need:
+        grown = torch.empty(need, dtype=torch.uint8, device=ws.device)
+        grown[: ws.numel()].copy_(ws)
+        prepared.workspace = ws = grown
     with torch.cuda.device(q.device):
         lse_strides = (ctypes.c_int64 * 2)(*lse.stride()) if return_lse else None
         rc = lib.hbsa_fwd_run_lse(q.data_ptr(), k.data_ptr(), v.data_ptr(), out_run.data_ptr(),

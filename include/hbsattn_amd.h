@@ -92,6 +92,19 @@ size_t hbsa_fwd_workspace_bytes_dtype(int32_t dtype, int32_t total_q, int32_t to
                                       int32_t num_q_block, int32_t num_k_block);
 
 /*
+ * Extra bytes, behind the hbsa_fwd_workspace_bytes_dtype(...) bytes of the same workspace, that let
+ * hbsa_fwd / hbsa_fwd_run split the work over key blocks when there are too few (kv head, q block)
+ * work items to fill the current device (short query side, long key side): every item is cut
+ * into up to 32 parts over its k blocks, the parts run as separate work items and a merge kernel
+ * combines their normalised partial results through their log-sum-exps.  0 when the split would
+ * not be used for this shape on this device.  A workspace without these bytes is valid; the call
+ * then runs unsplit.  The reference has no counterpart (one program per q tile,
+ * reference hbsattn/fwd_triton_auto_tile_size.py:283).
+ */
+size_t hbsa_fwd_split_workspace_bytes(int32_t total_q, int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+                                      int32_t num_q_block, int32_t num_k_block, int32_t q_block_size);
+
+/*
  * Block-sparse attention forward.  Replaces `_forward_auto_tile_size` and
  * `_forward_fix_tile_size` + their Triton `_fwd_kernel`s (reference
  * hbsattn/fwd_triton_auto_tile_size.py:76-310, hbsattn/fwd_triton_fix_tile_size.py:30-276).

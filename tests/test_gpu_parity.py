@@ -152,7 +152,8 @@ def test_full_size_properties_config2():
 
 
 def test_gqa_equals_mha_on_repeated_kv_bitwise():
-    w = make_problem(seed=11, q_lens=[1000, 2100], k_lens=[1000, 2100], hq=8, hk=2, d=128, qbs=64, kbs=128, keep=0.4,
+    # (enough work items that neither call is split over key blocks: the two would split differently)
+    w = make_problem(seed=11, q_lens=[3000, 4100], k_lens=[3000, 4100], hq=8, hk=2, d=128, qbs=64, kbs=128, keep=0.4,
                      diag=True, causal=True, scale=None)
     out = _run(w)
     k_rep, v_rep = w.k.repeat_interleave(4, 1), w.v.repeat_interleave(4, 1)
@@ -247,7 +248,7 @@ def test_calculate_blocks_on_device_matches_cpu():
 # ---------------------------------------------------------------------------------------
 # the combined C entry point, called the way a foreign binding would
 # ---------------------------------------------------------------------------------------
-def _call_hbsa_fwd(w, workspace_bytes=None, headdim=None):
+def _call_hbsa_fwd(w, workspace_bytes=None, headdim=None, split_room=False):
     import ctypes
 
     from hbsattn_amd import _lib
@@ -262,6 +263,9 @@ def _call_hbsa_fwd(w, workspace_bytes=None, headdim=None):
     code = _dtype_code(w.q.dtype)
     need = lib.hbsa_fwd_workspace_bytes_dtype(code, w.q.shape[0], w.k.shape[0], w.q.shape[1], w.k.shape[1], w.q.shape[2],
                                               nqb, nkb)
+    if split_room:   # room for the split over key blocks, like the operator provides it
+        need += lib.hbsa_fwd_split_workspace_bytes(w.q.shape[0], w.q.shape[1], w.k.shape[1], w.q.shape[2], nqb, nkb,
+                                                   w.q_block_size)
     ws = torch.empty(need, dtype=torch.uint8, device=w.q.device)
     strides = (ctypes.c_int64 * 11)(w.q.stride(0), w.q.stride(1), w.k.stride(0), w.k.stride(1), w.v.stride(0),
                                     w.v.stride(1), out.stride(0), out.stride(1), *w.block_mask.stride())
@@ -281,7 +285,7 @@ def _call_hbsa_fwd(w, workspace_bytes=None, headdim=None):
 def test_combined_c_entry_point_matches_operator_and_oracle(dtype):
     w = make_problem(seed=21, q_lens=[700, 1300, 64], k_lens=[900, 1300, 200], hq=8, hk=4, d=64, qbs=48, kbs=80, keep=0.4,
                      diag=True, causal=True, scale=0.2, dtype=dtype)
-    rc, out, _ = _call_hbsa_fwd(w)
+    rc, out, _ = _call_hbsa_fwd(w, split_room=True)
     assert rc == 0
     assert torch.equal(out, _run(w))
     assert_close_to_oracle(out, oracle_for(w), "hbsa_fwd")
@@ -349,7 +353,7 @@ def test_fp32_strided_inputs_headdim_padding_and_zero_tensor(fp32_mode):
 def test_fp32_through_the_combined_c_entry_point(fp32_mode):
     w = make_problem(seed=34, q_lens=[500, 64], k_lens=[700, 64], hq=4, hk=4, d=32, qbs=48, kbs=80, keep=0.5, diag=True,
                      causal=True, scale=None, dtype=torch.float32)
-    rc, out, _ = _call_hbsa_fwd(w)
+    rc, out, _ = _call_hbsa_fwd(w, split_room=True)
     assert rc == 0
     assert torch.equal(out, _run(w))
     assert_close_to_oracle(out, oracle_for(w), "hbsa_fwd fp32")
@@ -478,3 +482,28 @@ def test_strided_output_through_the_c_entry_point():
     assert rc == 0, _lib.last_error()
     assert torch.equal(out, _run(w))
     assert (wide[:, :, :16] == 7).all() and (wide[:, :, 80:] == 7).all()
+
+
+# ---------------------------------------------------------------------------------------
+# split over key blocks: few work items with long key sides
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,d,causal,kbs", [(torch.bfloat16, 128, True, 128), (torch.float16, 64, False, 48),
+                                                (torch.bfloat16, 32, True, 64)])
+def test_few_long_items_are_split_over_key_blocks_and_merged(dtype, d, causal, kbs):
+    from hbsattn_amd import _lib
+    w = make_problem(seed=81, q_lens=[128, 70], k_lens=[9000, 4000], hq=4, hk=2, d=d, qbs=64, kbs=kbs, keep=0.6, diag=True,
+                     causal=causal, scale=None, dtype=dtype)
+    lib = _lib.load()
+    extra = lib.hbsa_fwd_split_workspace_bytes(w.q.shape[0], 4, 2, d, w.q_meta[0], w.k_meta[0], 64)
+    assert extra > 0                                              # 8 work items on a 256-CU device: the split is used
+    out, lse = _run_lse(w)
+    ref_out, ref_lse = hbsa_oracle(w.q.cpu(), w.k.cpu(), w.v.cpu(), w.cu_q, w.cu_k, w.block_mask.cpu(), w.q_block_size,
+                                   w.k_block_size, w.causal, w.softmax_scale, return_lse=True)
+    assert_close_to_oracle(out, ref_out, "split")
+    assert (lse.cpu() - ref_lse).abs().max().item() <= 2e-3
+    assert torch.equal(out, _run(w))                              # deterministic, with and without the lse output
+    # the same call through the C entry point with a workspace that has no room for the split: unsplit path
+    rc, unsplit, _ = _call_hbsa_fwd(w)
+    assert rc == 0
+    assert_close_to_oracle(unsplit, ref_out, "unsplit")
+    assert (unsplit.float() - out.float()).abs().max().item() <= 2e-2
