@@ -84,11 +84,24 @@ def _check_block_sizes(q_block_size, k_block_size):
         "q_block_size and k_block_size must be integer multiples of 16."
 
 
+def _run_workspace_bytes(lib, device, code, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block, num_k_block,
+                         q_block_size) -> int:
+    """Bytes ``hbsa_fwd_run`` can use for one call: the work description, fp16 staging copies (fast
+    fp32 mode) and room for the split over key blocks the library uses when the work items cannot
+    fill the device."""
+    need = int(lib.hbsa_fwd_workspace_bytes_dtype(code, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
+                                                  num_k_block))
+    with torch.cuda.device(device):
+        need += int(lib.hbsa_fwd_split_workspace_bytes(total_q, nhead_q, nhead_k, headdim, num_q_block, num_k_block,
+                                                       q_block_size))
+    return need
+
+
 def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, num_q_block,
-                 q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, staging=None) -> PreparedMask:
-    """Runs the pre-pass kernel (``hbsa_fwd_prepare``) on the current stream.  ``staging`` =
-    ``(total_q, total_k, nhead_q, headdim)`` reserves the room fp32 q/k/v of that size need behind
-    the work description (``hbsa_run`` grows the workspace itself when it is missing)."""
+                 q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, run_shape=None) -> PreparedMask:
+    """Runs the pre-pass kernel (``hbsa_fwd_prepare``) on the current stream.  ``run_shape`` =
+    ``(dtype, total_q, total_k, nhead_q, headdim)`` of the q/k/v the mask will be used with sizes the
+    workspace for them at once (``hbsa_run`` grows it otherwise)."""
     if not block_mask.is_cuda:
         raise RuntimeError("hbsattn_amd runs on MI355X only: block_mask must be a CUDA(HIP) tensor; there is no CPU path")
     _check_block_sizes(q_block_size, k_block_size)
@@ -96,10 +109,12 @@ def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_s
     dev = block_mask.device
     nhead_k = block_mask.shape[0]
     ws_bytes = int(lib.hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block))
-    if staging is not None:
-        total_q, total_k, nhead_q, headdim = staging
-        ws_bytes = int(lib.hbsa_fwd_workspace_bytes_dtype(_lib.DTYPE_F32_STAGED16, total_q, total_k, nhead_q, nhead_k,
-                                                          headdim, num_q_block, num_k_block))
+    if run_shape is not None:
+        dtype, total_q, total_k, nhead_q, headdim = run_shape
+        d_run = next((d for d in _NATIVE_HEADDIMS if d >= headdim), headdim)
+        if dtype in _DTYPE_CODES and total_q > 0 and nhead_q > 0:
+            ws_bytes = max(ws_bytes, _run_workspace_bytes(lib, dev, _dtype_code(dtype), total_q, total_k, nhead_q, nhead_k,
+                                                          d_run, num_q_block, num_k_block, q_block_size))
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     cu_q, cu_k = _as_int32(cu_q_seqlens), _as_int32(cu_k_seqlens)
     qb2b, cu_nqb, cu_nkb = _as_int32(q_block_to_batch), _as_int32(cu_num_q_block), _as_int32(cu_num_k_block)
@@ -157,13 +172,8 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = 
                                    out_run.stride(0), out_run.stride(1))
     ws = prepared.workspace
     code = _dtype_code(q.dtype)
-    # room behind the work description for fp16 staging copies (fast fp32 mode) and for the split over
-    # key blocks the library uses when the work items cannot fill the device
-    need = int(lib.hbsa_fwd_workspace_bytes_dtype(code, total_q, total_k, nhead_q, nhead_k, d_run,
-                                                  prepared.num_q_block, prepared.num_k_block))
-    with torch.cuda.device(q.device):
-        need += int(lib.hbsa_fwd_split_workspace_bytes(total_q, nhead_q, nhead_k, d_run, prepared.num_q_block,
-                                                       prepared.num_k_block, prepared.q_block_size))
+    need = _run_workspace_bytes(lib, q.device, code, total_q, total_k, nhead_q, nhead_k, d_run, prepared.num_q_block,
+                                prepared.num_k_block, prepared.q_block_size)
     if ws.numel() < need:
         grown = torch.empty(need, dtype=torch.uint8, device=ws.device)
         grown[: ws.numel()].copy_(ws)
@@ -193,11 +203,9 @@ def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, 
     if block_mask.device != q.device:
         raise RuntimeError("q, k, v and block_mask must live on the same device")
     assert q.shape[1] % k.shape[1] == 0, "nhead_q must be divisible by nhead_k (for GQA)"
-    staging = None
-    if q.dtype == torch.float32 and _fp32_mode == "fast" and q.dim() == 3 and k.dim() == 3:
-        staging = (q.shape[0], k.shape[0], q.shape[1], next((d for d in _NATIVE_HEADDIMS if d >= q.shape[2]), q.shape[2]))
+    run_shape = (q.dtype, q.shape[0], k.shape[0], q.shape[1], q.shape[2]) if q.dim() == 3 and k.dim() == 3 else None
     prepared = hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, num_q_block,
-                            q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, staging)
+                            q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, run_shape)
     return hbsa_run(q, k, v, prepared, softmax_scale)
 
 
