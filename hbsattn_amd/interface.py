@@ -84,16 +84,25 @@ def _check_block_sizes(q_block_size, k_block_size):
         "q_block_size and k_block_size must be integer multiples of 16."
 
 
+_ws_bytes_cache = {}
+
+
 def _run_workspace_bytes(lib, device, code, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block, num_k_block,
                          q_block_size) -> int:
     """Bytes ``hbsa_fwd_run`` can use for one call: the work description, fp16 staging copies (fast
     fp32 mode) and room for the split over key blocks the library uses when the work items cannot
-    fill the device."""
-    need = int(lib.hbsa_fwd_workspace_bytes_dtype(code, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
-                                                  num_k_block))
-    with torch.cuda.device(device):
-        need += int(lib.hbsa_fwd_split_workspace_bytes(total_q, nhead_q, nhead_k, headdim, num_q_block, num_k_block,
-                                                       q_block_size))
+    fill the device.  Pure functions of the shape and the device, so the answers are kept."""
+    key = (device.index, code, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block, num_k_block, q_block_size)
+    need = _ws_bytes_cache.get(key)
+    if need is None:
+        need = int(lib.hbsa_fwd_workspace_bytes_dtype(code, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
+                                                      num_k_block))
+        with torch.cuda.device(device):
+            need += int(lib.hbsa_fwd_split_workspace_bytes(total_q, nhead_q, nhead_k, headdim, num_q_block, num_k_block,
+                                                           q_block_size))
+        if len(_ws_bytes_cache) > 4096:
+            _ws_bytes_cache.clear()
+        _ws_bytes_cache[key] = need
     return need
 
 
