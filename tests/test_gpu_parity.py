@@ -507,3 +507,13 @@ def test_few_long_items_are_split_over_key_blocks_and_merged(dtype, d, causal, k
     assert rc == 0
     assert_close_to_oracle(unsplit, ref_out, "unsplit")
     assert (unsplit.float() - out.float()).abs().max().item() <= 2e-2
+
+
+def test_split_with_many_kv_heads_and_a_head_count_that_is_no_multiple_of_eight():
+    w = make_problem(seed=82, q_lens=[64, 33], k_lens=[5000, 2500], hq=24, hk=12, d=64, qbs=64, kbs=128, keep=0.5, diag=True,
+                     causal=True, scale=0.1)
+    out, lse = _run_lse(w)
+    ref_out, ref_lse = hbsa_oracle(w.q.cpu(), w.k.cpu(), w.v.cpu(), w.cu_q, w.cu_k, w.block_mask.cpu(), w.q_block_size,
+                                   w.k_block_size, w.causal, w.softmax_scale, return_lse=True)
+    assert_close_to_oracle(out, ref_out, "split hk=12")
+    assert (lse.cpu() - ref_lse).abs().max().item() <= 2e-3

@@ -75,3 +75,18 @@ def test_cpu_tensors_are_refused_not_computed():
 def test_backward_is_not_implemented():
     with pytest.raises(NotImplementedError, match="gradient"):
         _HBSAttentionFunction.backward(None, None)
+
+
+def test_fp32_mode_switch_validates_and_returns_the_previous_mode():
+    import pytest
+    from hbsattn_amd import set_fp32_mode
+    from hbsattn_amd import interface
+    first = set_fp32_mode("fast")
+    try:
+        assert interface._fp32_mode == "fast"
+        assert set_fp32_mode("exact") == "fast"
+        with pytest.raises(ValueError):
+            set_fp32_mode("tf32")
+        assert interface._fp32_mode == "exact"
+    finally:
+        set_fp32_mode(first)
