@@ -333,7 +333,7 @@ def test_fp32_inputs_keep_their_range(q_mag, k_mag, v_mag, fp32_mode):
     out = _run(w).double().cpu() / v_mag
     sel = ~torch.isnan(base)
     err = (out[sel] - base.double()[sel]).abs()
-    tol = (2e-5, 2e-6) if fp32_mode == "exact" else (4e-3, 3e-4)
+    tol = (1e-4, 1e-5) if fp32_mode == "exact" else (4e-3, 3e-4)
     assert err.max().item() <= tol[0] and err.mean().item() <= tol[1], (err.max().item(), err.mean().item())
 
 
@@ -517,3 +517,42 @@ def test_split_with_many_kv_heads_and_a_head_count_that_is_no_multiple_of_eight(
                                    w.k_block_size, w.causal, w.softmax_scale, return_lse=True)
     assert_close_to_oracle(out, ref_out, "split hk=12")
     assert (lse.cpu() - ref_lse).abs().max().item() <= 2e-3
+
+
+# ---------------------------------------------------------------------------------------
+# seeded random shapes: lengths, head counts, block sizes, head dims, dtypes, masks
+# ---------------------------------------------------------------------------------------
+def test_seeded_random_shapes_against_the_oracle():
+    import random
+    rng = random.Random(2024)
+    from hbsattn_amd import set_fp32_mode
+    previous = set_fp32_mode("exact")
+    try:
+        for case in range(48):
+            batch = rng.randint(1, 4)
+            q_lens = [rng.randint(1, 700) for _ in range(batch)]
+            same = rng.random() < 0.3
+            k_lens = q_lens if same else [rng.randint(1, 900) for _ in range(batch)]
+            hk = rng.choice([1, 2, 3, 5, 9])
+            ratio = rng.choice([1, 1, 2, 4, 7])
+            d = rng.choice([16, 24, 32, 40, 64, 72, 96, 128])
+            qbs = 16 * rng.randint(1, 12)
+            kbs = 16 * rng.randint(1, 12)
+            dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+            causal = rng.random() < 0.6
+            scale = rng.choice([None, None, 0.05, 0.7])
+            keep = rng.choice([0.15, 0.5, 0.9, 1.0])
+            w = make_problem(seed=9000 + case, q_lens=q_lens, k_lens=k_lens, hq=hk * ratio, hk=hk, d=d, qbs=qbs, kbs=kbs,
+                             keep=keep, diag=rng.random() < 0.5, causal=causal, scale=scale, dtype=dtype)
+            what = (f"case {case}: q={q_lens} k={k_lens} heads={hk * ratio}/{hk} d={d} blocks={qbs}x{kbs} {dtype} "
+                    f"causal={causal} scale={scale} keep={keep}")
+            out, lse = _run_lse(w)
+            ref_out, ref_lse = hbsa_oracle(w.q.cpu(), w.k.cpu(), w.v.cpu(), w.cu_q, w.cu_k, w.block_mask.cpu(), qbs, kbs,
+                                           causal, scale, return_lse=True)
+            assert_close_to_oracle(out, ref_out, what)
+            lse = lse.cpu()
+            empty = torch.isinf(ref_lse)
+            assert torch.equal(torch.isinf(lse) & (lse < 0), empty), what
+            assert (lse[~empty] - ref_lse[~empty]).abs().max().item() <= 3e-3 if (~empty).any() else True, what
+    finally:
+        set_fp32_mode(previous)
