@@ -1044,14 +1044,20 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
               *(f32x4 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 4) = w;
             }
         } else {
+          // A lane holds dims 8*i4 + 4*g32 .. +3 of its row; lanes i and i+32 (same row) trade halves so
+          // that each stores 16 contiguous bytes: half the store instructions and write requests.
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-              u32x2 w;
-              w.x = E::pack2(o[dt][4 * i4 + 0] * inv, o[dt][4 * i4 + 1] * inv);
-              w.y = E::pack2(o[dt][4 * i4 + 2] * inv, o[dt][4 * i4 + 3] * inv);
-              *(u32x2 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 2) = w;
+            for (int m = 0; m < 2; ++m) {
+              const uint32_t ax = E::pack2(o[dt][8 * m + 0] * inv, o[dt][8 * m + 1] * inv);
+              const uint32_t ay = E::pack2(o[dt][8 * m + 2] * inv, o[dt][8 * m + 3] * inv);
+              const uint32_t bx = E::pack2(o[dt][8 * m + 4] * inv, o[dt][8 * m + 5] * inv);
+              const uint32_t by = E::pack2(o[dt][8 * m + 6] * inv, o[dt][8 * m + 7] * inv);
+              const auto rx = __builtin_amdgcn_permlane32_swap(ax, bx, false, false);
+              const auto ry = __builtin_amdgcn_permlane32_swap(ay, by, false, false);
+              const u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+              *(u32x4 *)(orow + (dt * 32 + 16 * m + 8 * g32) * 2) = w;
             }
         }
       }
