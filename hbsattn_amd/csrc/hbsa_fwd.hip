@@ -322,11 +322,6 @@ __global__ __launch_bounds__(256) void hbsa_f32_stage_kernel(F32Tensor t, const 
   }
 }
 
-#ifndef HBSA_INTERLEAVE_C
-#define HBSA_INTERLEAVE_C
-#define HBSA_INTERLEAVE_D
-#endif
-
 constexpr int kListCap = 1024;   // tile entries per list; longer items are expanded in chunks
 
 // Item header in LDS (16 ints).
@@ -684,6 +679,41 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     return p.q + (int64_t)(row_begin + r) * p.q_s + (int64_t)hq * p.q_h + g32 * 16;
   };
 
+  // Q^T fragments (B operand) of one item: lane (l32, g32) ends up with, per k-step ks, the 16 bytes
+  // d = 16*ks + 8*g32 .. +7 of query row l32.  Fetched so that four lanes read 64 contiguous bytes
+  // of a row (16 rows per instruction instead of 32, half the memory requests): with h = bit 4 of
+  // the lane, load A_k takes row (lane % 16), load B_k row 16 + (lane % 16), both at bytes
+  // 64*k + 32*h + 16*g32; then the h = 1 lanes of A_k and the h = 0 lanes of B_k trade places
+  // (v_permlane16_swap), which leaves k-step 2k in A_k and k-step 2k+1 in B_k.
+  short8v qf[KSTEPS];
+  auto load_q = [&](int hk, int sub, int row_begin, int rows) {
+    const int slot = sub * 4 + wave;
+    const int head_in_group = slot / p.wps;
+    const int row0 = (slot % p.wps) * kWaveRows;
+    if (head_in_group >= p.ratio || rows - row0 <= 0) return;   // this wavefront has no rows: qf is never used
+    const int hq = hk * p.ratio + head_in_group;
+    const char *base = p.q + (int64_t)hq * p.q_h + (lane & 16) * 2 + g32 * 16;
+    const int l16 = lane & 15;
+    const char *ra = base + (int64_t)(row_begin + min(row0 + l16, rows - 1)) * p.q_s;
+    const char *rb = base + (int64_t)(row_begin + min(row0 + 16 + l16, rows - 1)) * p.q_s;
+    if constexpr (KSTEPS >= 2) {
+#pragma unroll
+      for (int k = 0; k < KSTEPS / 2; ++k) {
+        u32x4 a = *(const u32x4 *)(ra + 64 * k), b = *(const u32x4 *)(rb + 64 * k);
+        a ^= p.q_sign;
+        b ^= p.q_sign;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const auto r = __builtin_amdgcn_permlane16_swap(a[j], b[j], false, false);
+          a[j] = r[0];
+          b[j] = r[1];
+        }
+        qf[2 * k] = __builtin_bit_cast(short8v, a);
+        qf[2 * k + 1] = __builtin_bit_cast(short8v, b);
+      }
+    }
+  };
+
   // ------------------------------------------------------------------ first item
   int c = 0;   // list / header of the current item
   if (hdr_word(0, H_HK) < 0) return;
@@ -696,19 +726,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
       issue_loads(0, tile_ptr(p.k + (int64_t)hk * p.k_h, tok, ks32), tile_ptr(p.v + (int64_t)hk * p.v_h, tok, vs32), (e & 63) + 1);
     }
   }
-  short8v qf[KSTEPS];   // Q^T fragments (B operand): lane holds query l32, d = 16*ks + 8*g32 .. +7
-  {
-    bool act; int hq, row0, nrows;
-    const char *qrow = q_row_ptr(hdr_word(0, H_HK), hdr_word(0, H_SUB), hdr_word(0, H_ROW_BEGIN), hdr_word(0, H_ROWS), act,
-                                 hq, row0, nrows);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      u32x4 raw = {0u, 0u, 0u, 0u};
-      if (act) raw = *(const u32x4 *)(qrow + ks * 32);
-      raw ^= p.q_sign;
-      qf[ks] = __builtin_bit_cast(short8v, raw);
-    }
-  }
+  load_q(hdr_word(0, H_HK), hdr_word(0, H_SUB), hdr_word(0, H_ROW_BEGIN), hdr_word(0, H_ROWS));
 
   for (;;) {   // ------------------------------------------------------ one iteration per work item
     const int cur_hk = hdr_word(c, H_HK);
@@ -918,7 +936,6 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
           read_vgroup(std::integral_constant<int, 0>{}, vb[0]);
           read_vgroup(std::integral_constant<int, 1>{}, vb[1]);
           half_exp(s0, p0a, p0b);
-          HBSA_INTERLEAVE_C
 
           // ---- row max of S1.  P0 was formed under the running max as it stood after S0 and is not
           // accumulated yet, so if that max has to move now (rare), P0 is rescaled along with O and l.
@@ -961,7 +978,6 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
           pv_group(p0b, vb[1]);
           read_vgroup(std::integral_constant<int, 3>{}, vb[1]);
           half_exp(s1, p1a, p1b);
-          HBSA_INTERLEAVE_D
 
           // ---- O^T += V^T[:, 32:64] . P1
           wait_vgroup(std::integral_constant<int, 2 * DT>{}, vb[0]);
@@ -972,16 +988,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         if (last && nxt_hk >= 0) {
           // Q of this item is no longer needed: fetch the next item's rows while the last MFMAs
           // drain and the epilogue runs
-          bool act; int hq1, r01, nr1;
-          const char *qrow = q_row_ptr(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS), act,
-                                       hq1, r01, nr1);
-#pragma unroll
-          for (int ks = 0; ks < KSTEPS; ++ks) {
-            u32x4 raw = {0u, 0u, 0u, 0u};
-            if (act) raw = *(const u32x4 *)(qrow + ks * 32);
-            raw ^= p.q_sign;
-            qf[ks] = __builtin_bit_cast(short8v, raw);
-          }
+          load_q(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS));
         }
         flip_buffers();
       }
@@ -1078,16 +1085,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
           issue_loads(buf, tile_ptr(p.k + (int64_t)nxt_hk * p.k_h, tok, ks32), tile_ptr(p.v + (int64_t)nxt_hk * p.v_h, tok, vs32),
                       (e1 & 63) + 1);
         }
-        bool act; int hq1, r01, nr1;
-        const char *qrow = q_row_ptr(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS), act,
-                                     hq1, r01, nr1);
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          u32x4 raw = {0u, 0u, 0u, 0u};
-          if (act) raw = *(const u32x4 *)(qrow + ks * 32);
-          raw ^= p.q_sign;
-          qf[ks] = __builtin_bit_cast(short8v, raw);
-        }
+        load_q(nxt_hk, hdr_word(c ^ 1, H_SUB), hdr_word(c ^ 1, H_ROW_BEGIN), hdr_word(c ^ 1, H_ROWS));
       }
       __syncthreads();   // wave 0 rewrites this item's list next; every wave has read its header by now
     }
