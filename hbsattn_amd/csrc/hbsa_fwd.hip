@@ -1039,9 +1039,9 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         const float lse = l_tot > 0.f ? (m_run * sm_c + __builtin_amdgcn_logf(l_tot)) * 0.69314718055994531f : -INFINITY;
         p.lse[(int64_t)(row_begin + row0 + l32) * p.lse_s + (int64_t)hq * p.lse_h] = lse;
       }
-      if (l32 < nrows) {
-        char *orow = p.out + (int64_t)(row_begin + row0 + l32) * p.o_s + (int64_t)hq * p.o_h;
-        if constexpr (OUT32) {
+      if constexpr (OUT32) {
+        if (l32 < nrows) {
+          char *orow = p.out + (int64_t)(row_begin + row0 + l32) * p.o_s + (int64_t)hq * p.o_h;
           const float f = inv * sm_out_mul;
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt)
@@ -1050,22 +1050,38 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
               f32x4 w = {o[dt][4 * i4 + 0] * f, o[dt][4 * i4 + 1] * f, o[dt][4 * i4 + 2] * f, o[dt][4 * i4 + 3] * f};
               *(f32x4 *)(orow + (dt * 32 + 8 * i4 + 4 * g32) * 4) = w;
             }
-        } else {
-          // A lane holds dims 8*i4 + 4*g32 .. +3 of its row; lanes i and i+32 (same row) trade halves so
-          // that each stores 16 contiguous bytes: half the store instructions and write requests.
+        }
+      } else {
+        // A lane holds dims 8*i4 + 4*g32 .. +3 of row l32, per 32-dim block.  Two exchanges turn that
+        // into 64 contiguous bytes of a row across four lanes, so that one store instruction covers
+        // 16 rows instead of 32 and the memory system sees a quarter of the write requests:
+        // lanes i and i+32 (same row) trade halves (16 contiguous bytes per lane), then lanes with
+        // bit 4 clear / set (rows l and 16 + l) trade the two 16-dim halves of the block.
+        const int l16 = lane & 15;
+        char *row_x = p.out + (int64_t)(row_begin + row0 + l16) * p.o_s + (int64_t)hq * p.o_h + (lane & 16) * 2 + g32 * 16;
+        char *row_y = row_x + (int64_t)16 * p.o_s;
+        const bool st_x = l16 < nrows, st_y = 16 + l16 < nrows;
 #pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt) {
+          u32x4 w[2];
 #pragma unroll
-            for (int m = 0; m < 2; ++m) {
-              const uint32_t ax = E::pack2(o[dt][8 * m + 0] * inv, o[dt][8 * m + 1] * inv);
-              const uint32_t ay = E::pack2(o[dt][8 * m + 2] * inv, o[dt][8 * m + 3] * inv);
-              const uint32_t bx = E::pack2(o[dt][8 * m + 4] * inv, o[dt][8 * m + 5] * inv);
-              const uint32_t by = E::pack2(o[dt][8 * m + 6] * inv, o[dt][8 * m + 7] * inv);
-              const auto rx = __builtin_amdgcn_permlane32_swap(ax, bx, false, false);
-              const auto ry = __builtin_amdgcn_permlane32_swap(ay, by, false, false);
-              const u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
-              *(u32x4 *)(orow + (dt * 32 + 16 * m + 8 * g32) * 2) = w;
-            }
+          for (int m = 0; m < 2; ++m) {
+            const uint32_t ax = E::pack2(o[dt][8 * m + 0] * inv, o[dt][8 * m + 1] * inv);
+            const uint32_t ay = E::pack2(o[dt][8 * m + 2] * inv, o[dt][8 * m + 3] * inv);
+            const uint32_t bx = E::pack2(o[dt][8 * m + 4] * inv, o[dt][8 * m + 5] * inv);
+            const uint32_t by = E::pack2(o[dt][8 * m + 6] * inv, o[dt][8 * m + 7] * inv);
+            const auto rx = __builtin_amdgcn_permlane32_swap(ax, bx, false, false);
+            const auto ry = __builtin_amdgcn_permlane32_swap(ay, by, false, false);
+            w[m] = u32x4{(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const auto r = __builtin_amdgcn_permlane16_swap(w[0][j], w[1][j], false, false);
+            w[0][j] = r[0];
+            w[1][j] = r[1];
+          }
+          if (st_x) *(u32x4 *)(row_x + dt * 64) = w[0];
+          if (st_y) *(u32x4 *)(row_y + dt * 64) = w[1];
         }
       }
       }
