@@ -48,7 +48,7 @@ BOUND = {"C2": "hbm", "T": "mfma", "C3": "mfma", "C4": "mfma", "C5": "hbm"}
 # (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, scaled by what the same counters read for a
 # 1 GiB device-to-device copy: factors 2.000 and 1.000).  Not measured live: a counter run needs
 # the profiler.  The summaries are under profiles/.
-MEASURED_TRAFFIC_BYTES = {"C2": 4.91e9, "T": 56.7e9}
+MEASURED_TRAFFIC_BYTES = {"C2": 4.87e9, "T": 56.6e9}
 
 
 def time_steps(fn, steps, warmup):
