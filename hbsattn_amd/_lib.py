@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhbsattn_amd.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 DTYPE_BF16 = 0
 DTYPE_F16 = 1
@@ -56,6 +56,11 @@ def load() -> ctypes.CDLL:
     lib.hbsa_fwd_split_workspace_bytes.argtypes = [ctypes.c_int32] * 7
     lib.hbsa_calculate_blocks.restype = ctypes.c_int
     lib.hbsa_calculate_blocks.argtypes = [vp, ctypes.c_int32, ctypes.c_int32, vp, vp, vp, vp, ctypes.c_int32]
+    lib.hbsa_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.hbsa_bwd_workspace_bytes.argtypes = [ctypes.c_int32] * 2
+    lib.hbsa_bwd.restype = ctypes.c_int
+    lib.hbsa_bwd.argtypes = ([vp] * 13 + [ctypes.c_size_t, vp, ctypes.c_size_t] + [ctypes.c_int32] * 12
+                             + [ctypes.c_float, i64p, vp])
     _lib = lib
     return lib
 

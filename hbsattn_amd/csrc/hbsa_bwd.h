@@ -1,0 +1,394 @@
+// Block-sparse attention backward for gfx950: dQ, dK, dV from dO, the forward's output and its
+// log-sum-exp.  Part of the translation unit hbsa_fwd.hip (included after the forward's helpers).
+//
+// The reference stops at the forward (reference hbsattn/hbsa_interface.py:31-32 raises
+// NotImplementedError in backward), so this follows the mathematics of that forward
+// (reference hbsattn/reference.py:23-107): with S = scale * Q K^T masked like the forward,
+// P = exp(S - lse), delta = rowsum(dO * O):
+//     dV = P^T dO      dP = dO V^T      dS = P * (dP - delta)
+//     dQ = scale * dS K                 dK = scale * dS^T Q
+//
+// Three kernels, no atomics, every output element written by exactly one workgroup:
+//   hbsa_bwd_delta_kernel : delta[row, q head] = sum_d dO * O
+//   hbsa_bwd_dq_kernel    : one workgroup per (kv head, q block, group of four 32-row wave slots), the
+//                           forward's decomposition; walks the kept k blocks of the q block's bit row.
+//                           Per 64-key tile  S^T = K Q^T,  dP^T = V dO^T  (A = tile rows from LDS,
+//                           B = Q^T / dO^T in registers),  dS^T in the accumulator layout is the B
+//                           operand of  dQ^T += K^T dS^T  (A = K^T through transposing LDS reads).
+//   hbsa_bwd_dkv_kernel   : the same with the roles of queries and keys exchanged: one workgroup per
+//                           (kv head, k block, group of four 32-key slots); K^T and V^T stay in
+//                           registers, the Q and dO rows of every q block that keeps the k block (and of
+//                           every q head of the group) stream through LDS in 64-row tiles:
+//                           S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS.
+// Both recompute S.  Tiles are loaded with plain global loads and two barriers per tile; a tile
+// that is read both by rows and transposed is stored twice, once in each of the forward's two
+// swizzled layouts.  This is the first correct version: the forward's persistent scheduling,
+// LDS-DMA and double buffering are not applied here yet.
+
+namespace {
+
+struct BwdParams {
+  const char *q, *k, *v, *dout;
+  char *dq, *dk, *dv;
+  const float *lse, *delta;   // [total_q, nhead_q], contiguous
+  const QBlockInfo *info;
+  const uint32_t *bits;
+  const int32_t *cu_k, *cu_num_q_block, *cu_num_k_block;
+  int64_t q_s, q_h, k_s, k_h, v_s, v_h, do_s, do_h, dq_s, dq_h, dk_s, dk_h, dv_s, dv_h;   // bytes
+  int32_t nqb, batch, ratio, nhead_q, kbs, wpr, causal;
+  int32_t wps, nsub;     // q side: wave slots per q head and workgroups per (kv head, q block), as in the forward
+  int32_t nsub_k;        // k side: workgroups per (kv head, k block) = ceil(k_block_size / 128)
+  float c;               // softmax_scale * log2(e), signed
+  float scale;
+};
+
+struct DeltaParams {
+  const char *out, *dout;
+  float *delta;
+  int64_t o_s, o_h, do_s, do_h;   // bytes
+  int32_t total_q, nhead_q;
+};
+
+// delta[row, head] = sum over d of dO * O; one thread per (row, head)
+template <int D, typename E>
+__global__ __launch_bounds__(256) void hbsa_bwd_delta_kernel(DeltaParams p) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)p.total_q * p.nhead_q) return;
+  const int64_t row = i / p.nhead_q;
+  const int h = (int)(i - row * p.nhead_q);
+  const char *o = p.out + row * p.o_s + h * p.o_h;
+  const char *g = p.dout + row * p.do_s + h * p.do_h;
+  float acc = 0.f;
+#pragma unroll
+  for (int ch = 0; ch < D / 8; ++ch) {
+    const u32x4 a = *(const u32x4 *)(o + ch * 16), b = *(const u32x4 *)(g + ch * 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc += E::lo(a[j]) * E::lo(b[j]);
+      acc += E::hi(a[j]) * E::hi(b[j]);
+    }
+  }
+  p.delta[i] = acc;
+}
+
+// ---- shared pieces of the two main kernels ---------------------------------------------------------
+template <int D>
+struct BwdTile {
+  static constexpr int RB = D * 2;            // row bytes
+  static constexpr int CPR = RB / 16;         // 16-byte chunks per row
+  static constexpr int RPG = 16 / CPR > 0 ? 16 / CPR : 1;
+  static constexpr int TILE_BYTES = 64 * RB;
+  static constexpr int KSTEPS = D / 16;
+  static constexpr int DT = D / 32;
+  // chunk swizzles of the forward's K tile (read by rows) and V tile (read transposed)
+  static __device__ __forceinline__ int swz_rows(int r) { return (r / RPG) % CPR; }
+  static __device__ __forceinline__ int swz_tr(int r) { return CPR >= 8 ? (((r / RPG) % (CPR / 4)) << 2) : 0; }
+};
+
+// 64 rows of `src` (row stride `stride` bytes, rows past `valid` repeat the last valid one) into LDS:
+// `by_rows` in the layout read by rows, `transposed` (may be null) in the layout read transposed.
+template <int D>
+__device__ __forceinline__ void bwd_load_tile(const char *src, int64_t stride, int valid, char *by_rows, char *transposed) {
+  using T = BwdTile<D>;
+#pragma unroll
+  for (int i = 0; i < 64 * T::CPR / 256; ++i) {
+    const int ch = i * 256 + threadIdx.x;
+    const int r = ch / T::CPR, pc = ch % T::CPR;
+    const u32x4 x = *(const u32x4 *)(src + (int64_t)min(r, valid - 1) * stride + pc * 16);
+    *(u32x4 *)(by_rows + r * T::RB + ((pc ^ T::swz_rows(r)) << 4)) = x;
+    if (transposed != nullptr) *(u32x4 *)(transposed + r * T::RB + ((pc ^ T::swz_tr(r)) << 4)) = x;
+  }
+}
+
+// acc[h] (h = 0, 1: rows 0-31 / 32-63 of the tile) = tile rows . frag^T, the forward's S^T = K Q^T
+template <int D, typename E>
+__device__ __forceinline__ void bwd_rows_times_frag(const char *tile, const short8v *frag, int lane, f32x16 &a0, f32x16 &a1) {
+  using T = BwdTile<D>;
+  const int l32 = lane & 31, g32 = lane >> 5;
+  const int rd = l32 * T::RB + ((g32 ^ T::swz_rows(l32)) << 4);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) { a0[i] = 0.f; a1[i] = 0.f; }
+#pragma unroll
+  for (int ks = 0; ks < T::KSTEPS; ++ks) {
+    const short8v x0 = *(const short8v *)(tile + (rd ^ (ks * 32)));
+    const short8v x1 = *(const short8v *)(tile + (rd ^ (ks * 32)) + 32 * T::RB);
+    a0 = E::mfma(x0, frag[ks], a0);
+    a1 = E::mfma(x1, frag[ks], a1);
+  }
+}
+
+// acc[dt] += tile^T (rows 16*g .. 16*g+15 of the tile as the contraction index) . packed, the forward's
+// O^T += V^T P^T for one group of 16 keys
+template <int D, typename E>
+__device__ __forceinline__ void bwd_transposed_times_packed(const char *tile, int g, short8v packed, int lane, f32x16 *acc) {
+  using T = BwdTile<D>;
+  const int g32 = lane >> 5;
+  const int key = 4 * g32 + ((lane & 15) >> 2);
+  const int lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+  const int rd = key * T::RB + ((lc | T::swz_tr(key)) << 4) + 8 * (lane & 1);
+#pragma unroll
+  for (int dt = 0; dt < T::DT; ++dt) {
+    const char *a = tile + (rd ^ (dt * 64)) + g * 16 * T::RB;
+    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(a));
+    const short4v hi =
+        __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(a + 8 * T::RB));
+    const short8v va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    acc[dt] = E::mfma(va, packed, acc[dt]);
+  }
+}
+
+// 16 accumulator values of one lane -> two B operands (rows 0-15 and 16-31 of the half tile)
+template <typename E>
+__device__ __forceinline__ void bwd_pack(const float *e, short8v &lo, short8v &hi) {
+  u32x4 w[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) w[j][q4] = E::pack2(e[8 * j + 2 * q4], e[8 * j + 2 * q4 + 1]);
+  lo = __builtin_bit_cast(short8v, w[0]);
+  hi = __builtin_bit_cast(short8v, w[1]);
+}
+
+// accumulators [d, row = lane % 32] * f -> out row (16-bit), the forward's plain epilogue
+template <int D, typename E>
+__device__ __forceinline__ void bwd_store_rows(char *row_ptr, const f32x16 *acc, float f, int g32) {
+#pragma unroll
+  for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      u32x2 w;
+      w.x = E::pack2(acc[dt][4 * i4 + 0] * f, acc[dt][4 * i4 + 1] * f);
+      w.y = E::pack2(acc[dt][4 * i4 + 2] * f, acc[dt][4 * i4 + 3] * f);
+      *(u32x2 *)(row_ptr + (dt * 32 + 8 * i4 + 4 * g32) * 2) = w;
+    }
+}
+
+// ---- dQ ----------------------------------------------------------------------------------------------
+template <int D, typename E>
+__global__ __launch_bounds__(kThreads, 1) void hbsa_bwd_dq_kernel(BwdParams p) {
+  using T = BwdTile<D>;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  char *k_rows = lds, *k_tr = lds + T::TILE_BYTES, *v_rows = lds + 2 * T::TILE_BYTES;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g32 = lane >> 5, l32 = lane & 31;
+  const int hk = blockIdx.y;
+  const int qb = blockIdx.x / p.nsub, sub = blockIdx.x - qb * p.nsub;
+  const QBlockInfo inf = p.info[qb];
+
+  const int slot = sub * 4 + wave;
+  const int head_in_group = slot / p.wps;
+  const int row0 = (slot % p.wps) * kWaveRows;
+  const int nrows = min(kWaveRows, inf.rows - row0);
+  const bool active = head_in_group < p.ratio && nrows > 0;
+  const int hq = hk * p.ratio + head_in_group;
+
+  short8v qf[T::KSTEPS], dof[T::KSTEPS];   // Q^T and dO^T fragments: lane holds row l32, d = 16*ks + 8*g32 .. +7
+  float lse2 = INFINITY, dlt = 0.f;         // a row that takes no part gets P = exp2(-inf) = 0
+  const int my_row = inf.row_begin + min(row0 + l32, inf.rows - 1);
+  if (active) {
+    const char *qrow = p.q + (int64_t)my_row * p.q_s + (int64_t)hq * p.q_h + g32 * 16;
+    const char *grow = p.dout + (int64_t)my_row * p.do_s + (int64_t)hq * p.do_h + g32 * 16;
+#pragma unroll
+    for (int ks = 0; ks < T::KSTEPS; ++ks) {
+      qf[ks] = *(const short8v *)(qrow + ks * 32);
+      dof[ks] = *(const short8v *)(grow + ks * 32);
+    }
+    const float l = p.lse[(int64_t)my_row * p.nhead_q + hq];
+    lse2 = l == -INFINITY ? INFINITY : l * kLog2e;
+    dlt = p.delta[(int64_t)my_row * p.nhead_q + hq];
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < T::KSTEPS; ++ks) { qf[ks] = short8v{0, 0, 0, 0, 0, 0, 0, 0}; dof[ks] = qf[ks]; }
+  }
+  f32x16 acc[T::DT];
+#pragma unroll
+  for (int dt = 0; dt < T::DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
+
+  const int lane_kvis = inf.q_pos + min(row0 + l32, inf.rows - 1) + inf.shift;   // last key position the row sees (causal)
+  const uint32_t *bits = p.bits + ((size_t)hk * p.nqb + qb) * p.wpr;
+  const char *kg = p.k + (int64_t)hk * p.k_h + (int64_t)inf.key_begin * p.k_s;
+  const char *vg = p.v + (int64_t)hk * p.v_h + (int64_t)inf.key_begin * p.v_s;
+
+  for (int j = 0; j < inf.nkblk; ++j) {
+    if (((bits[j >> 5] >> (j & 31)) & 1u) == 0) continue;
+    const int kend = min((j + 1) * p.kbs, inf.kmax);
+    for (int kpos = j * p.kbs; kpos < kend; kpos += kTileKeys) {
+      const int valid = min(kTileKeys, kend - kpos);
+      __syncthreads();   // the previous tile has been read by every wavefront
+      bwd_load_tile<D>(kg + (int64_t)kpos * p.k_s, p.k_s, valid, k_rows, k_tr);
+      bwd_load_tile<D>(vg + (int64_t)kpos * p.v_s, p.v_s, valid, v_rows, nullptr);
+      __syncthreads();
+      if (!active) continue;
+      f32x16 s[2], dp[2];
+      bwd_rows_times_frag<D, E>(k_rows, qf, lane, s[0], s[1]);
+      bwd_rows_times_frag<D, E>(v_rows, dof, lane, dp[0], dp[1]);
+      int lim = valid;   // keys of the tile below lim are visible to this lane's row
+      if (p.causal) lim = min(lim, lane_kvis - kpos + 1);
+      lim -= 4 * g32;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        float e[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const bool vis = 32 * h + 8 * (i >> 2) + (i & 3) < lim;
+          const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[h][i], p.c, -lse2)) : 0.f;
+          e[i] = pv * (dp[h][i] - dlt);
+        }
+        short8v lo, hi;
+        bwd_pack<E>(e, lo, hi);
+        bwd_transposed_times_packed<D, E>(k_tr, 2 * h, lo, lane, acc);
+        bwd_transposed_times_packed<D, E>(k_tr, 2 * h + 1, hi, lane, acc);
+      }
+    }
+  }
+  if (active && l32 < nrows)
+    bwd_store_rows<D, E>(p.dq + (int64_t)(inf.row_begin + row0 + l32) * p.dq_s + (int64_t)hq * p.dq_h, acc, p.scale, g32);
+}
+
+// ---- dK, dV ------------------------------------------------------------------------------------------
+template <int D, typename E>
+__global__ __launch_bounds__(kThreads, 1) void hbsa_bwd_dkv_kernel(BwdParams p) {
+  using T = BwdTile<D>;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  char *q_rows = lds, *q_tr = lds + T::TILE_BYTES, *g_rows = lds + 2 * T::TILE_BYTES, *g_tr = lds + 3 * T::TILE_BYTES;
+  float *lse_s = (float *)(lds + 4 * T::TILE_BYTES);   // [64] log2-domain log-sum-exp of the tile's rows
+  float *dlt_s = lse_s + 64;                           // [64] their delta
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g32 = lane >> 5, l32 = lane & 31;
+  const int hk = blockIdx.y;
+  const int kb = blockIdx.x / p.nsub_k, sub = blockIdx.x - kb * p.nsub_k;
+
+  int b = 0;   // the sequence the k block belongs to
+  while (b + 1 < p.batch && p.cu_num_k_block[b + 1] <= kb) ++b;
+  const int kbl = kb - p.cu_num_k_block[b];          // in-sequence index of the k block
+  const int k0 = p.cu_k[b], klen = p.cu_k[b + 1] - k0;
+  const int krows = min(p.kbs, klen - kbl * p.kbs);  // keys in the block
+  const int row0 = (sub * 4 + wave) * kWaveRows;
+  const int nrows = min(kWaveRows, krows - row0);
+  const bool active = nrows > 0;
+  const int key_pos = kbl * p.kbs + min(row0 + l32, krows - 1);   // in-sequence position of this lane's key
+  const int wg_first_key = kbl * p.kbs + sub * 4 * kWaveRows;     // of the workgroup's first key
+
+  short8v kf[T::KSTEPS], vf[T::KSTEPS];   // K^T and V^T fragments: lane holds key l32, d = 16*ks + 8*g32 .. +7
+  if (active) {
+    const char *krow = p.k + (int64_t)(k0 + key_pos) * p.k_s + (int64_t)hk * p.k_h + g32 * 16;
+    const char *vrow = p.v + (int64_t)(k0 + key_pos) * p.v_s + (int64_t)hk * p.v_h + g32 * 16;
+#pragma unroll
+    for (int ks = 0; ks < T::KSTEPS; ++ks) {
+      kf[ks] = *(const short8v *)(krow + ks * 32);
+      vf[ks] = *(const short8v *)(vrow + ks * 32);
+    }
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < T::KSTEPS; ++ks) { kf[ks] = short8v{0, 0, 0, 0, 0, 0, 0, 0}; vf[ks] = kf[ks]; }
+  }
+  f32x16 acc_k[T::DT], acc_v[T::DT];
+#pragma unroll
+  for (int dt = 0; dt < T::DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { acc_k[dt][i] = 0.f; acc_v[dt][i] = 0.f; }
+
+  for (int qb = p.cu_num_q_block[b]; qb < p.cu_num_q_block[b + 1]; ++qb) {
+    const uint32_t word = p.bits[((size_t)hk * p.nqb + qb) * p.wpr + (kbl >> 5)];
+    if (((word >> (kbl & 31)) & 1u) == 0) continue;
+    const QBlockInfo inf = p.info[qb];
+    for (int r = 0; r < p.ratio; ++r) {
+      const int hq = hk * p.ratio + r;
+      for (int qoff = 0; qoff < inf.rows; qoff += 64) {
+        const int valid = min(64, inf.rows - qoff);
+        // causal: none of the tile's rows sees any key of this workgroup
+        if (p.causal && inf.q_pos + qoff + valid - 1 + inf.shift < wg_first_key) continue;
+        const int64_t row_first = inf.row_begin + qoff;
+        __syncthreads();   // the previous tile has been read by every wavefront
+        bwd_load_tile<D>(p.q + row_first * p.q_s + (int64_t)hq * p.q_h, p.q_s, valid, q_rows, q_tr);
+        bwd_load_tile<D>(p.dout + row_first * p.do_s + (int64_t)hq * p.do_h, p.do_s, valid, g_rows, g_tr);
+        if (threadIdx.x < 64) {
+          const int rr = threadIdx.x;
+          float l2 = INFINITY, dl = 0.f;   // rows past the block's end take no part
+          if (rr < valid) {
+            const float l = p.lse[(row_first + rr) * p.nhead_q + hq];
+            l2 = l == -INFINITY ? INFINITY : l * kLog2e;
+            dl = p.delta[(row_first + rr) * p.nhead_q + hq];
+          }
+          lse_s[rr] = l2;
+          dlt_s[rr] = dl;
+        }
+        __syncthreads();
+        if (!active) continue;
+        f32x16 s[2], dp[2];
+        bwd_rows_times_frag<D, E>(q_rows, kf, lane, s[0], s[1]);
+        bwd_rows_times_frag<D, E>(g_rows, vf, lane, dp[0], dp[1]);
+        // query rows of the tile at or above lim see this lane's key (causal); lanes past the block's keys see nothing
+        int first_vis = 0;
+        if (p.causal) first_vis = max(0, key_pos - inf.shift - (inf.q_pos + qoff));
+        if (l32 >= nrows) first_vis = 64;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          float ep[16], ed[16];
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            const int rr0 = 32 * h + 8 * a + 4 * g32;
+            const f32x4 l4 = *(const f32x4 *)(lse_s + rr0), d4 = *(const f32x4 *)(dlt_s + rr0);
+#pragma unroll
+            for (int bq = 0; bq < 4; ++bq) {
+              const int i = 4 * a + bq;
+              const bool vis = rr0 + bq >= first_vis;   // rows past `valid` carry lse = +inf, hence P = 0
+              const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[h][i], p.c, -l4[bq])) : 0.f;
+              ep[i] = pv;
+              ed[i] = pv * (dp[h][i] - d4[bq]);
+            }
+          }
+          short8v plo, phi, dlo, dhi;
+          bwd_pack<E>(ep, plo, phi);
+          bwd_pack<E>(ed, dlo, dhi);
+          bwd_transposed_times_packed<D, E>(g_tr, 2 * h, plo, lane, acc_v);
+          bwd_transposed_times_packed<D, E>(g_tr, 2 * h + 1, phi, lane, acc_v);
+          bwd_transposed_times_packed<D, E>(q_tr, 2 * h, dlo, lane, acc_k);
+          bwd_transposed_times_packed<D, E>(q_tr, 2 * h + 1, dhi, lane, acc_k);
+        }
+      }
+    }
+  }
+  if (active && l32 < nrows) {
+    const int64_t row = k0 + kbl * p.kbs + row0 + l32;
+    bwd_store_rows<D, E>(p.dk + row * p.dk_s + (int64_t)hk * p.dk_h, acc_k, p.scale, g32);
+    bwd_store_rows<D, E>(p.dv + row * p.dv_s + (int64_t)hk * p.dv_h, acc_v, 1.f, g32);
+  }
+}
+
+template <int D, typename E>
+int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_k_block, hipStream_t stream) {
+  using T = BwdTile<D>;
+  const int64_t rows = (int64_t)dp.total_q * dp.nhead_q;
+  hipLaunchKernelGGL((hbsa_bwd_delta_kernel<D, E>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream, dp);
+  const int lds_dq = 3 * T::TILE_BYTES, lds_dkv = 4 * T::TILE_BYTES + 512;
+  if (lds_dkv > 48 * 1024) {
+    static thread_local bool raised[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+      return fail(HBSA_ERR_UNSUPPORTED, "no current device, or device index above %d", kMaxDevices - 1);
+    if (!raised[dev]) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&hbsa_bwd_dkv_kernel<D, E>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv);
+      if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(&hbsa_bwd_dq_kernel<D, E>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_dq);
+      if (e != hipSuccess) return (int)e;
+      raised[dev] = true;
+    }
+  }
+  hipLaunchKernelGGL((hbsa_bwd_dq_kernel<D, E>), dim3((unsigned)(bp.nqb * bp.nsub), (unsigned)nhead_k), dim3(kThreads), lds_dq,
+                     stream, bp);
+  hipLaunchKernelGGL((hbsa_bwd_dkv_kernel<D, E>), dim3((unsigned)(num_k_block * bp.nsub_k), (unsigned)nhead_k), dim3(kThreads),
+                     lds_dkv, stream, bp);
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : (int)e;
+}
+
+}  // namespace

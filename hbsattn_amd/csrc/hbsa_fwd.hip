@@ -171,9 +171,9 @@ struct ElemBF16 {
     bf16x2 v = {(__bf16)lo, (__bf16)hi};
     return __builtin_bit_cast(uint32_t, v);
   }
-  static __device__ __forceinline__ uint32_t scale_packed(uint32_t w, float f) {
-    return pack2(__builtin_bit_cast(float, w << 16) * f, __builtin_bit_cast(float, w & 0xffff0000u) * f);
-  }
+  static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+  static __device__ __forceinline__ uint32_t scale_packed(uint32_t w, float f) { return pack2(lo(w) * f, hi(w) * f); }
   // acc + lo + hi of a packed pair (v_dot2c_f32_bf16 with a vector of ones)
   static __device__ __forceinline__ float dot2_ones(uint32_t packed, float acc) {
     const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
@@ -188,10 +188,9 @@ struct ElemF16 {
     f16x2 v = {(_Float16)lo, (_Float16)hi};
     return __builtin_bit_cast(uint32_t, v);
   }
-  static __device__ __forceinline__ uint32_t scale_packed(uint32_t w, float f) {
-    const f16x2 v = __builtin_bit_cast(f16x2, w);
-    return pack2((float)v.x * f, (float)v.y * f);
-  }
+  static __device__ __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w).x; }
+  static __device__ __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w).y; }
+  static __device__ __forceinline__ uint32_t scale_packed(uint32_t w, float f) { return pack2(lo(w) * f, hi(w) * f); }
   static __device__ __forceinline__ float dot2_ones(uint32_t packed, float acc) {
     const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, packed), ones, acc, false);
@@ -1483,6 +1482,8 @@ int launch_fwd_f32(const FwdParams &fp, float c_signed, long long items, hipStre
 
 }  // namespace
 
+#include "hbsa_bwd.h"
+
 extern "C" {
 
 int hbsa_abi_version(void) { return HBSA_ABI_VERSION; }
@@ -1745,4 +1746,74 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32
                       num_q_block, num_k_block, q_block_size, k_block_size, causal, softmax_scale, strides, stream);
 }
 
+
+size_t hbsa_bwd_workspace_bytes(int32_t total_q, int32_t nhead_q) {
+  if (total_q < 0 || nhead_q < 0) return 0;
+  return align_up((size_t)total_q * nhead_q * sizeof(float), 256);
+}
+
+int hbsa_bwd(const void *q, const void *k, const void *v, const void *out, const void *dout, const float *lse, void *dq,
+             void *dk, void *dv, const int32_t *cu_k_seqlens, const int32_t *cu_num_q_block, const int32_t *cu_num_k_block,
+             const void *workspace, size_t workspace_bytes, void *bwd_workspace, size_t bwd_workspace_bytes, int32_t dtype,
+             int32_t batch, int32_t total_q, int32_t total_k, int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+             int32_t num_q_block, int32_t num_k_block, int32_t q_block_size, int32_t k_block_size, int32_t causal,
+             float softmax_scale, const int64_t *strides, void *stream) {
+  g_err[0] = 0;
+  if (!q || !k || !v || !out || !dout || !lse || !dq || !dk || !dv || !cu_k_seqlens || !cu_num_q_block || !cu_num_k_block ||
+      !workspace || !bwd_workspace || !strides)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer argument");
+  if (dtype != HBSA_DTYPE_BF16 && dtype != HBSA_DTYPE_F16)
+    return fail(HBSA_ERR_UNSUPPORTED, "the backward takes bf16 or fp16 tensors (dtype code %d given)", dtype);
+  if (headdim != 32 && headdim != 64 && headdim != 128) return fail(HBSA_ERR_UNSUPPORTED, "headdim %d not in {32, 64, 128}", headdim);
+  if (batch <= 0 || total_q < 0 || total_k < 0 || nhead_q <= 0 || nhead_k <= 0 || nhead_q % nhead_k != 0 || num_q_block < 0 ||
+      num_k_block < 0)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "bad sizes");
+  if (q_block_size <= 0 || k_block_size <= 0 || q_block_size % 16 || k_block_size % 16)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "q_block_size and k_block_size must be positive multiples of 16");
+  for (int i = 0; i < 16; ++i)
+    if (strides[i] % 8 != 0)
+      return fail(HBSA_ERR_INVALID_ARGUMENT, "stride %d (%lld elements) is not a multiple of 8 (16-byte rows)", i,
+                  (long long)strides[i]);
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)dout | (uintptr_t)dq | (uintptr_t)dk |
+       (uintptr_t)dv) & 15)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "q/k/v/out/dout/dq/dk/dv must be 16-byte aligned");
+  if ((uintptr_t)workspace & 255) return fail(HBSA_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
+  if (workspace_bytes < hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block))
+    return fail(HBSA_ERR_WORKSPACE_TOO_SMALL, "workspace smaller than hbsa_fwd_workspace_bytes");
+  if (((uintptr_t)bwd_workspace & 15) || bwd_workspace_bytes < hbsa_bwd_workspace_bytes(total_q, nhead_q))
+    return fail(HBSA_ERR_WORKSPACE_TOO_SMALL, "bwd_workspace smaller than hbsa_bwd_workspace_bytes, or not 16-byte aligned");
+  if (total_q == 0 || total_k == 0 || num_q_block == 0 || num_k_block == 0) return 0;
+
+  const int es = 2;
+  BwdParams bp;
+  std::memset(&bp, 0, sizeof(bp));
+  bp.q = (const char *)q; bp.k = (const char *)k; bp.v = (const char *)v; bp.dout = (const char *)dout;
+  bp.dq = (char *)dq; bp.dk = (char *)dk; bp.dv = (char *)dv;
+  bp.lse = lse; bp.delta = (const float *)bwd_workspace;
+  bp.info = (const QBlockInfo *)workspace;
+  bp.bits = (const uint32_t *)((const char *)workspace + bits_offset(num_q_block));
+  bp.cu_k = cu_k_seqlens; bp.cu_num_q_block = cu_num_q_block; bp.cu_num_k_block = cu_num_k_block;
+  bp.q_s = strides[0] * es; bp.q_h = strides[1] * es; bp.k_s = strides[2] * es; bp.k_h = strides[3] * es;
+  bp.v_s = strides[4] * es; bp.v_h = strides[5] * es; bp.do_s = strides[8] * es; bp.do_h = strides[9] * es;
+  bp.dq_s = strides[10] * es; bp.dq_h = strides[11] * es; bp.dk_s = strides[12] * es; bp.dk_h = strides[13] * es;
+  bp.dv_s = strides[14] * es; bp.dv_h = strides[15] * es;
+  bp.nqb = num_q_block; bp.batch = batch; bp.ratio = nhead_q / nhead_k; bp.nhead_q = nhead_q; bp.kbs = k_block_size;
+  bp.wpr = words_per_row(num_k_block); bp.causal = causal ? 1 : 0;
+  bp.wps = (q_block_size + kWaveRows - 1) / kWaveRows;
+  bp.nsub = (bp.ratio * bp.wps + 3) / 4;
+  bp.nsub_k = (k_block_size + 4 * kWaveRows - 1) / (4 * kWaveRows);
+  bp.c = softmax_scale * kLog2e;
+  bp.scale = softmax_scale;
+  DeltaParams dp;
+  dp.out = (const char *)out; dp.dout = (const char *)dout; dp.delta = (float *)bwd_workspace;
+  dp.o_s = strides[6] * es; dp.o_h = strides[7] * es; dp.do_s = strides[8] * es; dp.do_h = strides[9] * es;
+  dp.total_q = total_q; dp.nhead_q = nhead_q;
+  hipStream_t st = (hipStream_t)stream;
+  const bool bf = dtype == HBSA_DTYPE_BF16;
+  switch (headdim) {
+    case 32: return bf ? launch_bwd<32, ElemBF16>(bp, dp, nhead_k, num_k_block, st) : launch_bwd<32, ElemF16>(bp, dp, nhead_k, num_k_block, st);
+    case 64: return bf ? launch_bwd<64, ElemBF16>(bp, dp, nhead_k, num_k_block, st) : launch_bwd<64, ElemF16>(bp, dp, nhead_k, num_k_block, st);
+    default: return bf ? launch_bwd<128, ElemBF16>(bp, dp, nhead_k, num_k_block, st) : launch_bwd<128, ElemF16>(bp, dp, nhead_k, num_k_block, st);
+  }
+}
 }  // extern "C"

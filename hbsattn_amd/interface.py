@@ -69,8 +69,13 @@ class PreparedMask:
     combination: the device scratch the attention kernel reads.  Reusable across calls that
     share those, e.g. the layers of a model that share one sparsity pattern."""
 
-    def __init__(self, workspace, nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, causal):
+    def __init__(self, workspace, nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, causal,
+                 cu_k_seqlens=None, cu_num_q_block=None, cu_num_k_block=None):
         self.workspace = workspace
+        # int32 device tensors the backward reads besides the workspace
+        self.cu_k_seqlens = cu_k_seqlens
+        self.cu_num_q_block = cu_num_q_block
+        self.cu_num_k_block = cu_num_k_block
         self.nhead_k = nhead_k
         self.num_q_block = num_q_block
         self.num_k_block = num_k_block
@@ -135,7 +140,8 @@ def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_s
                                   torch.cuda.current_stream().cuda_stream)
     if rc != 0:
         raise RuntimeError(f"hbsa_fwd_prepare failed (code {rc}): {_lib.last_error()}")
-    return PreparedMask(workspace, nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, causal)
+    return PreparedMask(workspace, nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, causal, cu_k, cu_nqb,
+                        cu_nkb)
 
 
 def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = False):
@@ -203,8 +209,52 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = 
     return (out, lse) if return_lse else out
 
 
+def backward_supported(q: torch.Tensor) -> bool:
+    """The backward kernels take bf16 / fp16 tensors with a native head dim (32, 64 or 128)."""
+    return q.dtype in (torch.bfloat16, torch.float16) and q.dim() == 3 and q.shape[2] in _NATIVE_HEADDIMS
+
+
+def hbsa_backward(q, k, v, out, dout, lse, prepared: PreparedMask, softmax_scale):
+    """``(dq, dk, dv)`` through ``hbsa_bwd`` on the current stream.  ``out`` and ``lse`` are what
+    ``hbsa_run(..., return_lse=True)`` returned for the same q, k, v, prepared mask and scale."""
+    if not backward_supported(q):
+        raise NotImplementedError("hbsattn_amd: the backward takes bfloat16 / float16 tensors with headdim 32, 64 or 128")
+    if prepared.cu_k_seqlens is None:
+        raise ValueError("this PreparedMask was built without the sequence boundaries the backward needs")
+    lib = _lib.load()
+    total_q, nhead_q, headdim = q.shape
+    total_k, nhead_k = k.shape[0], k.shape[1]
+    scale = float(softmax_scale) if softmax_scale is not None else headdim ** -0.5
+    q = q if _rows_ok(q) else q.contiguous()
+    k = k if _rows_ok(k) else k.contiguous()
+    v = v if _rows_ok(v) else v.contiguous()
+    out = out if _rows_ok(out) else out.contiguous()
+    dout = dout if _rows_ok(dout) else dout.contiguous()
+    lse = lse.contiguous()
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if total_q == 0 or total_k == 0:
+        return dq.zero_(), dk.zero_(), dv.zero_()
+    bws_bytes = int(lib.hbsa_bwd_workspace_bytes(total_q, nhead_q))
+    bws = torch.empty(bws_bytes, dtype=torch.uint8, device=q.device)
+    strides = (ctypes.c_int64 * 16)(q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+                                    out.stride(0), out.stride(1), dout.stride(0), dout.stride(1), dq.stride(0),
+                                    dq.stride(1), dk.stride(0), dk.stride(1), dv.stride(0), dv.stride(1))
+    ws = prepared.workspace
+    with torch.cuda.device(q.device):
+        rc = lib.hbsa_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), lse.data_ptr(),
+                          dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), prepared.cu_k_seqlens.data_ptr(),
+                          prepared.cu_num_q_block.data_ptr(), prepared.cu_num_k_block.data_ptr(), ws.data_ptr(), ws.numel(),
+                          bws.data_ptr(), bws_bytes, _dtype_code(q.dtype), prepared.cu_k_seqlens.numel() - 1, total_q,
+                          total_k, nhead_q, nhead_k, headdim, prepared.num_q_block, prepared.num_k_block,
+                          prepared.q_block_size, prepared.k_block_size, int(prepared.causal), scale, strides,
+                          torch.cuda.current_stream().cuda_stream)
+    if rc != 0:
+        raise RuntimeError(f"hbsa_bwd failed (code {rc}): {_lib.last_error()}")
+    return dq, dk, dv
+
+
 def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, softmax_scale,
-                 num_q_block, q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block) -> torch.Tensor:
+                 num_q_block, q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, ctx=None) -> torch.Tensor:
     """Host launcher: checks, scratch allocation, pre-pass and attention kernel through the C ABI.
     No device synchronisation happens here."""
     if not q.is_cuda:
@@ -215,6 +265,13 @@ def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, 
     run_shape = (q.dtype, q.shape[0], k.shape[0], q.shape[1], q.shape[2]) if q.dim() == 3 and k.dim() == 3 else None
     prepared = hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, num_q_block,
                             q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, run_shape)
+    if ctx is not None and any(ctx.needs_input_grad[:3]) and backward_supported(q):
+        # keep what the backward needs: the log-sum-exp, the output and the prepared mask
+        out, lse = hbsa_run(q, k, v, prepared, softmax_scale, return_lse=True)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.prepared = prepared
+        ctx.softmax_scale = softmax_scale
+        return out
     return hbsa_run(q, k, v, prepared, softmax_scale)
 
 
@@ -245,11 +302,17 @@ class _HBSAttentionFunction(torch.autograd.Function):
             raise ValueError(f"Invalid tile mode: {tile_mode}")
         return hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal,
                             softmax_scale, int(num_q_block), q_block_to_batch, cu_num_q_block, int(num_k_block),
-                            cu_num_k_block)
+                            cu_num_k_block, ctx=ctx)
 
     @staticmethod
     def backward(ctx, do):
-        raise NotImplementedError("It does not support gradient propagation yet")
+        # The reference stops here (reference hbsattn/hbsa_interface.py:31-32 raises NotImplementedError);
+        # bf16 / fp16 inputs with a native head dim get their gradients, anything else still raises.
+        if getattr(ctx, "prepared", None) is None:
+            raise NotImplementedError("It does not support gradient propagation yet for this dtype / headdim")
+        q, k, v, out, lse = ctx.saved_tensors
+        dq, dk, dv = hbsa_backward(q, k, v, out, do, lse, ctx.prepared, ctx.softmax_scale)
+        return (dq, dk, dv) + (None,) * 16
 
 
 HBSAttention = _HBSAttentionFunction.apply

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define HBSA_ABI_VERSION 2
+#define HBSA_ABI_VERSION 3
 
 /* element types of q/k/v/out (reference: dtype follows the input tensors,
  * hbsattn/fwd_triton_auto_tile_size.py:272) */
@@ -194,6 +194,38 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out,
                      int32_t q_block_size, int32_t k_block_size,
                      int32_t causal, float softmax_scale,
                      const int64_t *strides, void *stream);
+
+/*
+ * Backward of the block-sparse attention forward: dq, dk, dv from dout = d loss / d out.
+ * The reference has no counterpart: its operator's backward raises NotImplementedError
+ * (reference hbsattn/hbsa_interface.py:31-32); the gradients are those of the forward the reference
+ * defines (reference hbsattn/reference.py:23-107).
+ *
+ *   q, out, dout, dq [total_q, nhead_q, headdim]     k, v, dk, dv [total_k, nhead_k, headdim]
+ *   lse         float [total_q, nhead_q], contiguous: what hbsa_fwd_run_lse wrote for the same
+ *               q/k/v, mask and softmax_scale
+ *   workspace   as left by hbsa_fwd_prepare (or hbsa_fwd) for the same mask, sequence boundaries,
+ *               block sizes and `causal`; read only
+ *   bwd_workspace  >= hbsa_bwd_workspace_bytes(total_q, nhead_q) bytes of device scratch, 16-byte aligned
+ *   strides     int64[16] = { q_tok, q_head, k_tok, k_head, v_tok, v_head, out_tok, out_head,
+ *                             dout_tok, dout_head, dq_tok, dq_head, dk_tok, dk_head, dv_tok, dv_head }
+ *
+ * Supported: HBSA_DTYPE_BF16 and HBSA_DTYPE_F16, headdim in {32, 64, 128}.  Every element of dq, dk
+ * and dv is written (zeros where no gradient flows); no atomics, so results are deterministic.
+ */
+size_t hbsa_bwd_workspace_bytes(int32_t total_q, int32_t nhead_q);
+
+int hbsa_bwd(const void *q, const void *k, const void *v, const void *out, const void *dout,
+             const float *lse, void *dq, void *dk, void *dv,
+             const int32_t *cu_k_seqlens, const int32_t *cu_num_q_block, const int32_t *cu_num_k_block,
+             const void *workspace, size_t workspace_bytes,
+             void *bwd_workspace, size_t bwd_workspace_bytes,
+             int32_t dtype, int32_t batch, int32_t total_q, int32_t total_k,
+             int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+             int32_t num_q_block, int32_t num_k_block,
+             int32_t q_block_size, int32_t k_block_size,
+             int32_t causal, float softmax_scale,
+             const int64_t *strides, void *stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,125 @@
+"""Backward parity on an MI355X: dq, dk, dv of the HIP kernels (through the C ABI, via the autograd
+operator) against the float32 gradient oracle (``oracle.grads``) on the same seeded inputs.
+
+The reference has no backward to compare with (reference ``hbsattn/hbsa_interface.py:31-32``); the
+oracle is pinned in ``tests/test_oracle_grads.py``.  Tolerance for 16-bit tensors against float32:
+max-abs error at most 1e-2 of the largest gradient magnitude (at least 1), mean-abs at most 2e-3.
+"""
+import pytest
+import torch
+
+from oracle.dense import hbsa_oracle
+from oracle.grads import hbsa_oracle_grads
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL_TOL = 1e-2
+MEAN_ABS_TOL = 2e-3
+
+
+def _problem(seed, q_lens, k_lens, hq, hk, d, qbs, kbs, keep, dtype):
+    from hbsattn_amd import calculate_blocks
+    g = torch.Generator().manual_seed(seed)
+    cu_q, cu_k = [0], [0]
+    for a, b in zip(q_lens, k_lens):
+        cu_q.append(cu_q[-1] + a)
+        cu_k.append(cu_k[-1] + b)
+    q = torch.randn(cu_q[-1], hq, d, generator=g).to(dtype)
+    k = torch.randn(cu_k[-1], hk, d, generator=g).to(dtype)
+    v = torch.randn(cu_k[-1], hk, d, generator=g).to(dtype)
+    do = torch.randn(cu_q[-1], hq, d, generator=g).to(dtype)
+    cq = torch.tensor(cu_q, dtype=torch.int32, device="cuda")
+    ck = torch.tensor(cu_k, dtype=torch.int32, device="cuda")
+    nq, nk = calculate_blocks(cq, qbs)[0], calculate_blocks(ck, kbs)[0]
+    mask = torch.rand(hk, nq, nk, generator=g) < keep
+    return q, k, v, do, cu_q, cu_k, cq, ck, mask
+
+
+def _gpu_grads(q, k, v, do, cq, ck, mask, qbs, kbs, causal, scale):
+    from hbsattn_amd import HBSAttention
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = HBSAttention(qd, kd, vd, cq, ck, mask.cuda(), qbs, kbs, causal, scale)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    return out.detach(), qd.grad, kd.grad, vd.grad
+
+
+def _check(got, ref, what):
+    got = got.float().cpu()
+    assert torch.isfinite(got).all(), f"{what}: non-finite gradient"
+    err = (got - ref).abs()
+    lim = MAX_REL_TOL * max(1.0, ref.abs().max().item())
+    assert err.max().item() <= lim, f"{what}: max-abs {err.max().item():.3e} > {lim:.3e}"
+    assert err.mean().item() <= MEAN_ABS_TOL, f"{what}: mean-abs {err.mean().item():.3e} > {MEAN_ABS_TOL}"
+
+
+CASES = [
+    # seed, q_lens, k_lens, hq, hk, d, qbs, kbs, keep, causal, scale
+    (1, [64], [64], 1, 1, 32, 32, 32, 1.1, False, None),
+    (2, [64], [64], 1, 1, 128, 32, 32, 1.1, True, None),
+    (3, [100, 37], [80, 130], 4, 2, 64, 32, 48, 0.6, True, None),
+    (4, [300, 129, 5], [257, 129, 70], 6, 2, 128, 128, 128, 0.5, False, None),
+    (5, [300, 129, 5], [257, 129, 70], 6, 2, 128, 64, 256, 0.5, True, 0.2),
+    (6, [512, 1000], [512, 1000], 8, 8, 128, 128, 128, 0.3, True, None),
+    (7, [200, 1], [1, 333], 8, 1, 64, 80, 48, 0.7, False, -0.1),
+    (8, [33, 77, 190], [190, 33, 77], 2, 2, 32, 16, 16, 0.4, True, None),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("case", CASES, ids=[f"case{c[0]}" for c in CASES])
+def test_gradients_match_oracle(case, dtype):
+    seed, q_lens, k_lens, hq, hk, d, qbs, kbs, keep, causal, scale = case
+    q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(seed, q_lens, k_lens, hq, hk, d, qbs, kbs, keep, dtype)
+    print(f"backward case {case} {dtype}", flush=True)
+    out, dq, dk, dv = _gpu_grads(q, k, v, do, cq, ck, mask, qbs, kbs, causal, scale)
+    ref_out = hbsa_oracle(q, k, v, cu_q, cu_k, mask, qbs, kbs, causal, scale)
+    assert (out.float().cpu() - ref_out).abs().max().item() <= 2e-2     # the forward that saved the log-sum-exp
+    rdq, rdk, rdv = hbsa_oracle_grads(q, k, v, do, cu_q, cu_k, mask, qbs, kbs, causal, scale)
+    _check(dq, rdq, "dq")
+    _check(dk, rdk, "dk")
+    _check(dv, rdv, "dv")
+
+
+def test_rows_without_visible_keys_and_unkept_keys_get_exact_zeros():
+    # q longer than k under bottom-right causal alignment: the first 32 rows see no key; k block 1 is kept by nobody
+    q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(11, [48], [32], 2, 1, 32, 16, 16, 1.1, torch.bfloat16)
+    mask[:, :, 1] = False
+    print("backward zero rows", flush=True)
+    _, dq, dk, dv = _gpu_grads(q, k, v, do, cq, ck, mask, 16, 16, True, None)
+    assert torch.count_nonzero(dq[:16]) == 0          # rows 0-15 see keys <= row - 16 < 0
+    assert torch.count_nonzero(dq[16:32]) > 0
+    assert torch.count_nonzero(dk[16:]) == 0 and torch.count_nonzero(dv[16:]) == 0
+    rdq, rdk, rdv = hbsa_oracle_grads(q, k, v, do, cu_q, cu_k, mask, 16, 16, True, None)
+    _check(dq, rdq, "dq")
+    _check(dk, rdk, "dk")
+    _check(dv, rdv, "dv")
+
+
+def test_backward_is_deterministic():
+    q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(12, [700, 300], [700, 300], 4, 2, 128, 128, 128, 0.5, torch.bfloat16)
+    print("backward determinism", flush=True)
+    a = _gpu_grads(q, k, v, do, cq, ck, mask, 128, 128, True, None)
+    b = _gpu_grads(q, k, v, do, cq, ck, mask, 128, 128, True, None)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+
+
+def test_gqa_gradients_equal_mha_with_repeated_kv_heads():
+    # one kv head shared by 4 q heads == 4 identical kv heads; dk, dv of the shared head are the sums over the copies
+    q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(13, [150, 90], [150, 90], 4, 1, 64, 32, 32, 0.6, torch.bfloat16)
+    print("backward gqa", flush=True)
+    _, dq, dk, dv = _gpu_grads(q, k, v, do, cq, ck, mask, 32, 32, True, None)
+    _, dq4, dk4, dv4 = _gpu_grads(q, k.repeat(1, 4, 1), v.repeat(1, 4, 1), do, cq, ck, mask.repeat(4, 1, 1), 32, 32, True, None)
+    assert torch.equal(dq, dq4)
+    torch.testing.assert_close(dk.float(), dk4.float().sum(dim=1, keepdim=True), atol=3e-2, rtol=2e-2)
+    torch.testing.assert_close(dv.float(), dv4.float().sum(dim=1, keepdim=True), atol=3e-2, rtol=2e-2)
+
+
+def test_float32_inputs_still_raise_like_the_reference():
+    from hbsattn_amd import HBSAttention
+    q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(14, [64], [64], 2, 2, 32, 32, 32, 1.1, torch.float32)
+    qd = q.cuda().requires_grad_(True)
+    out = HBSAttention(qd, k.cuda(), v.cuda(), cq, ck, mask.cuda(), 32, 32, False, None)
+    with pytest.raises(NotImplementedError):
+        out.backward(do.cuda())
