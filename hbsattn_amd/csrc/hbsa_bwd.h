@@ -20,10 +20,10 @@
 //                           registers, the Q and dO rows of every q block that keeps the k block (and of
 //                           every q head of the group) stream through LDS in 64-row tiles:
 //                           S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS.
-// Both recompute S.  Tiles are loaded with plain global loads and two barriers per tile; a tile
-// that is read both by rows and transposed is stored twice, once in each of the forward's two
-// swizzled layouts.  This is the first correct version: the forward's persistent scheduling,
-// LDS-DMA and double buffering are not applied here yet.
+// Both recompute S.  A tile goes from global memory to registers while the tile before it is computed
+// on, and from registers to LDS between two barriers; a tile that is read both by rows and transposed
+// is stored twice, once in each of the forward's two swizzled layouts.  The forward's persistent
+// scheduling and LDS-DMA double buffering are not applied here yet.
 
 namespace {
 
@@ -85,18 +85,35 @@ struct BwdTile {
   static __device__ __forceinline__ int swz_tr(int r) { return CPR >= 8 ? (((r / RPG) % (CPR / 4)) << 2) : 0; }
 };
 
-// 64 rows of `src` (row stride `stride` bytes, rows past `valid` repeat the last valid one) into LDS:
-// `by_rows` in the layout read by rows, `transposed` (may be null) in the layout read transposed.
+// A 64-row tile on its way from global memory to LDS: each thread holds LOADS 16-byte chunks.  The
+// fetch of the next tile is issued before the current one is computed on, so its latency hides
+// behind the matrix work; bwd_stash_tile writes the chunks to LDS once the buffers are free again.
 template <int D>
-__device__ __forceinline__ void bwd_load_tile(const char *src, int64_t stride, int valid, char *by_rows, char *transposed) {
+struct BwdTileRegs {
+  static constexpr int LOADS = 64 * BwdTile<D>::CPR / 256;
+  u32x4 x[LOADS];
+};
+// 64 rows of `src` (row stride `stride` bytes; rows past `valid` repeat the last valid one)
+template <int D>
+__device__ __forceinline__ void bwd_fetch_tile(const char *src, int64_t stride, int valid, BwdTileRegs<D> &t) {
   using T = BwdTile<D>;
 #pragma unroll
-  for (int i = 0; i < 64 * T::CPR / 256; ++i) {
+  for (int i = 0; i < BwdTileRegs<D>::LOADS; ++i) {
     const int ch = i * 256 + threadIdx.x;
     const int r = ch / T::CPR, pc = ch % T::CPR;
-    const u32x4 x = *(const u32x4 *)(src + (int64_t)min(r, valid - 1) * stride + pc * 16);
-    *(u32x4 *)(by_rows + r * T::RB + ((pc ^ T::swz_rows(r)) << 4)) = x;
-    if (transposed != nullptr) *(u32x4 *)(transposed + r * T::RB + ((pc ^ T::swz_tr(r)) << 4)) = x;
+    t.x[i] = *(const u32x4 *)(src + (int64_t)min(r, valid - 1) * stride + pc * 16);
+  }
+}
+// `by_rows`: the layout read by rows; `transposed` (may be null): the layout read transposed
+template <int D>
+__device__ __forceinline__ void bwd_stash_tile(const BwdTileRegs<D> &t, char *by_rows, char *transposed) {
+  using T = BwdTile<D>;
+#pragma unroll
+  for (int i = 0; i < BwdTileRegs<D>::LOADS; ++i) {
+    const int ch = i * 256 + threadIdx.x;
+    const int r = ch / T::CPR, pc = ch % T::CPR;
+    *(u32x4 *)(by_rows + r * T::RB + ((pc ^ T::swz_rows(r)) << 4)) = t.x[i];
+    if (transposed != nullptr) *(u32x4 *)(transposed + r * T::RB + ((pc ^ T::swz_tr(r)) << 4)) = t.x[i];
   }
 }
 
@@ -213,36 +230,58 @@ __global__ __launch_bounds__(kThreads, 1) void hbsa_bwd_dq_kernel(BwdParams p) {
   const char *kg = p.k + (int64_t)hk * p.k_h + (int64_t)inf.key_begin * p.k_s;
   const char *vg = p.v + (int64_t)hk * p.v_h + (int64_t)inf.key_begin * p.v_s;
 
-  for (int j = 0; j < inf.nkblk; ++j) {
-    if (((bits[j >> 5] >> (j & 31)) & 1u) == 0) continue;
-    const int kend = min((j + 1) * p.kbs, inf.kmax);
-    for (int kpos = j * p.kbs; kpos < kend; kpos += kTileKeys) {
-      const int valid = min(kTileKeys, kend - kpos);
-      __syncthreads();   // the previous tile has been read by every wavefront
-      bwd_load_tile<D>(kg + (int64_t)kpos * p.k_s, p.k_s, valid, k_rows, k_tr);
-      bwd_load_tile<D>(vg + (int64_t)kpos * p.v_s, p.v_s, valid, v_rows, nullptr);
-      __syncthreads();
-      if (!active) continue;
-      f32x16 s[2], dp[2];
-      bwd_rows_times_frag<D, E>(k_rows, qf, lane, s[0], s[1]);
-      bwd_rows_times_frag<D, E>(v_rows, dof, lane, dp[0], dp[1]);
-      int lim = valid;   // keys of the tile below lim are visible to this lane's row
-      if (p.causal) lim = min(lim, lane_kvis - kpos + 1);
-      lim -= 4 * g32;
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        float e[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const bool vis = 32 * h + 8 * (i >> 2) + (i & 3) < lim;
-          const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[h][i], p.c, -lse2)) : 0.f;
-          e[i] = pv * (dp[h][i] - dlt);
-        }
-        short8v lo, hi;
-        bwd_pack<E>(e, lo, hi);
-        bwd_transposed_times_packed<D, E>(k_tr, 2 * h, lo, lane, acc);
-        bwd_transposed_times_packed<D, E>(k_tr, 2 * h + 1, hi, lane, acc);
+  // the tile sequence: 64-key tiles of the kept k blocks, cut at the last key any row of the block sees
+  int j = -1, kpos = 0;
+  auto next_tile = [&]() -> bool {
+    if (j >= 0) {
+      kpos += kTileKeys;
+      if (kpos < min((j + 1) * p.kbs, inf.kmax)) return true;
+    }
+    for (++j; j < inf.nkblk; ++j)
+      if ((bits[j >> 5] >> (j & 31)) & 1u) {
+        kpos = j * p.kbs;   // below kmax: the pre-pass cleared the bits of blocks no row can see
+        return true;
       }
+    return false;
+  };
+  auto tile_valid = [&]() { return min(kTileKeys, min((j + 1) * p.kbs, inf.kmax) - kpos); };
+  BwdTileRegs<D> kt, vt;
+  bool have = next_tile();
+  if (have) {
+    bwd_fetch_tile<D>(kg + (int64_t)kpos * p.k_s, p.k_s, tile_valid(), kt);
+    bwd_fetch_tile<D>(vg + (int64_t)kpos * p.v_s, p.v_s, tile_valid(), vt);
+  }
+  while (have) {
+    const int cur_kpos = kpos, valid = tile_valid();
+    __syncthreads();   // the previous tile has been read by every wavefront
+    bwd_stash_tile<D>(kt, k_rows, k_tr);
+    bwd_stash_tile<D>(vt, v_rows, nullptr);
+    __syncthreads();
+    have = next_tile();
+    if (have) {   // on its way while this tile is computed on
+      bwd_fetch_tile<D>(kg + (int64_t)kpos * p.k_s, p.k_s, tile_valid(), kt);
+      bwd_fetch_tile<D>(vg + (int64_t)kpos * p.v_s, p.v_s, tile_valid(), vt);
+    }
+    if (!active) continue;
+    f32x16 s[2], dp[2];
+    bwd_rows_times_frag<D, E>(k_rows, qf, lane, s[0], s[1]);
+    bwd_rows_times_frag<D, E>(v_rows, dof, lane, dp[0], dp[1]);
+    int lim = valid;   // keys of the tile below lim are visible to this lane's row
+    if (p.causal) lim = min(lim, lane_kvis - cur_kpos + 1);
+    lim -= 4 * g32;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      float e[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const bool vis = 32 * h + 8 * (i >> 2) + (i & 3) < lim;
+        const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[h][i], p.c, -lse2)) : 0.f;
+        e[i] = pv * (dp[h][i] - dlt);
+      }
+      short8v lo, hi;
+      bwd_pack<E>(e, lo, hi);
+      bwd_transposed_times_packed<D, E>(k_tr, 2 * h, lo, lane, acc);
+      bwd_transposed_times_packed<D, E>(k_tr, 2 * h + 1, hi, lane, acc);
     }
   }
   if (active && l32 < nrows)
@@ -294,65 +333,96 @@ __global__ __launch_bounds__(kThreads, 1) void hbsa_bwd_dkv_kernel(BwdParams p) 
 #pragma unroll
     for (int i = 0; i < 16; ++i) { acc_k[dt][i] = 0.f; acc_v[dt][i] = 0.f; }
 
-  for (int qb = p.cu_num_q_block[b]; qb < p.cu_num_q_block[b + 1]; ++qb) {
-    const uint32_t word = p.bits[((size_t)hk * p.nqb + qb) * p.wpr + (kbl >> 5)];
-    if (((word >> (kbl & 31)) & 1u) == 0) continue;
-    const QBlockInfo inf = p.info[qb];
-    for (int r = 0; r < p.ratio; ++r) {
-      const int hq = hk * p.ratio + r;
-      for (int qoff = 0; qoff < inf.rows; qoff += 64) {
-        const int valid = min(64, inf.rows - qoff);
-        // causal: none of the tile's rows sees any key of this workgroup
-        if (p.causal && inf.q_pos + qoff + valid - 1 + inf.shift < wg_first_key) continue;
-        const int64_t row_first = inf.row_begin + qoff;
-        __syncthreads();   // the previous tile has been read by every wavefront
-        bwd_load_tile<D>(p.q + row_first * p.q_s + (int64_t)hq * p.q_h, p.q_s, valid, q_rows, q_tr);
-        bwd_load_tile<D>(p.dout + row_first * p.do_s + (int64_t)hq * p.do_h, p.do_s, valid, g_rows, g_tr);
-        if (threadIdx.x < 64) {
-          const int rr = threadIdx.x;
-          float l2 = INFINITY, dl = 0.f;   // rows past the block's end take no part
-          if (rr < valid) {
-            const float l = p.lse[(row_first + rr) * p.nhead_q + hq];
-            l2 = l == -INFINITY ? INFINITY : l * kLog2e;
-            dl = p.delta[(row_first + rr) * p.nhead_q + hq];
-          }
-          lse_s[rr] = l2;
-          dlt_s[rr] = dl;
-        }
-        __syncthreads();
-        if (!active) continue;
-        f32x16 s[2], dp[2];
-        bwd_rows_times_frag<D, E>(q_rows, kf, lane, s[0], s[1]);
-        bwd_rows_times_frag<D, E>(g_rows, vf, lane, dp[0], dp[1]);
-        // query rows of the tile at or above lim see this lane's key (causal); lanes past the block's keys see nothing
-        int first_vis = 0;
-        if (p.causal) first_vis = max(0, key_pos - inf.shift - (inf.q_pos + qoff));
-        if (l32 >= nrows) first_vis = 64;
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          float ep[16], ed[16];
-#pragma unroll
-          for (int a = 0; a < 4; ++a) {
-            const int rr0 = 32 * h + 8 * a + 4 * g32;
-            const f32x4 l4 = *(const f32x4 *)(lse_s + rr0), d4 = *(const f32x4 *)(dlt_s + rr0);
-#pragma unroll
-            for (int bq = 0; bq < 4; ++bq) {
-              const int i = 4 * a + bq;
-              const bool vis = rr0 + bq >= first_vis;   // rows past `valid` carry lse = +inf, hence P = 0
-              const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[h][i], p.c, -l4[bq])) : 0.f;
-              ep[i] = pv;
-              ed[i] = pv * (dp[h][i] - d4[bq]);
-            }
-          }
-          short8v plo, phi, dlo, dhi;
-          bwd_pack<E>(ep, plo, phi);
-          bwd_pack<E>(ed, dlo, dhi);
-          bwd_transposed_times_packed<D, E>(g_tr, 2 * h, plo, lane, acc_v);
-          bwd_transposed_times_packed<D, E>(g_tr, 2 * h + 1, phi, lane, acc_v);
-          bwd_transposed_times_packed<D, E>(q_tr, 2 * h, dlo, lane, acc_k);
-          bwd_transposed_times_packed<D, E>(q_tr, 2 * h + 1, dhi, lane, acc_k);
+  // the tile sequence: for every q block of the sequence that keeps this k block, for every q head of
+  // the group, the block's rows in 64-row tiles (under a causal mask only those with a row that sees a
+  // key of this workgroup)
+  int qb = p.cu_num_q_block[b] - 1, r = 0, qoff = 0;
+  const int qb_end = p.cu_num_q_block[b + 1];
+  QBlockInfo inf = {};
+  auto tile_reaches = [&]() {
+    return !p.causal || inf.q_pos + qoff + min(64, inf.rows - qoff) - 1 + inf.shift >= wg_first_key;
+  };
+  auto next_tile = [&]() -> bool {
+    for (;;) {
+      if (qb >= p.cu_num_q_block[b]) {   // inside a kept q block: next tile, then next head
+        qoff += 64;
+        if (qoff >= inf.rows) { qoff = 0; ++r; }
+        if (r < p.ratio) {
+          if (tile_reaches()) return true;
+          continue;
         }
       }
+      for (++qb; qb < qb_end; ++qb) {
+        const uint32_t word = p.bits[((size_t)hk * p.nqb + qb) * p.wpr + (kbl >> 5)];
+        if ((word >> (kbl & 31)) & 1u) break;
+      }
+      if (qb >= qb_end) return false;
+      inf = p.info[qb];
+      r = 0;
+      qoff = -64;   // the step above moves to the block's first tile
+    }
+  };
+  BwdTileRegs<D> qt, gt;
+  float l2_next = INFINITY, dl_next = 0.f;   // threads 0-63: log2-domain log-sum-exp and delta of the tile's row
+  auto fetch = [&]() {
+    const int valid = min(64, inf.rows - qoff);
+    const int64_t row_first = inf.row_begin + qoff;
+    const int hq = hk * p.ratio + r;
+    bwd_fetch_tile<D>(p.q + row_first * p.q_s + (int64_t)hq * p.q_h, p.q_s, valid, qt);
+    bwd_fetch_tile<D>(p.dout + row_first * p.do_s + (int64_t)hq * p.do_h, p.do_s, valid, gt);
+    l2_next = INFINITY;   // rows past the block's end take no part: P = exp2(-inf) = 0
+    dl_next = 0.f;
+    if (threadIdx.x < valid) {
+      const float l = p.lse[(row_first + threadIdx.x) * p.nhead_q + hq];
+      l2_next = l == -INFINITY ? INFINITY : l * kLog2e;
+      dl_next = p.delta[(row_first + threadIdx.x) * p.nhead_q + hq];
+    }
+  };
+  bool have = next_tile();
+  if (have) fetch();
+  while (have) {
+    const int first_q_pos = inf.q_pos + qoff, shift = inf.shift;
+    __syncthreads();   // the previous tile has been read by every wavefront
+    bwd_stash_tile<D>(qt, q_rows, q_tr);
+    bwd_stash_tile<D>(gt, g_rows, g_tr);
+    if (threadIdx.x < 64) {
+      lse_s[threadIdx.x] = l2_next;
+      dlt_s[threadIdx.x] = dl_next;
+    }
+    __syncthreads();
+    have = next_tile();
+    if (have) fetch();   // on its way while this tile is computed on
+    if (!active) continue;
+    f32x16 s[2], dp[2];
+    bwd_rows_times_frag<D, E>(q_rows, kf, lane, s[0], s[1]);
+    bwd_rows_times_frag<D, E>(g_rows, vf, lane, dp[0], dp[1]);
+    // rows of the tile from first_vis on see this lane's key (causal); lanes past the block's keys see nothing
+    int first_vis = 0;
+    if (p.causal) first_vis = max(0, key_pos - shift - first_q_pos);
+    if (l32 >= nrows) first_vis = 64;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      float ep[16], ed[16];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const int rr0 = 32 * h + 8 * a + 4 * g32;
+        const f32x4 l4 = *(const f32x4 *)(lse_s + rr0), d4 = *(const f32x4 *)(dlt_s + rr0);
+#pragma unroll
+        for (int bq = 0; bq < 4; ++bq) {
+          const int i = 4 * a + bq;
+          const bool vis = rr0 + bq >= first_vis;   // rows past the block's end carry lse = +inf, hence P = 0
+          const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[h][i], p.c, -l4[bq])) : 0.f;
+          ep[i] = pv;
+          ed[i] = pv * (dp[h][i] - d4[bq]);
+        }
+      }
+      short8v plo, phi, dlo, dhi;
+      bwd_pack<E>(ep, plo, phi);
+      bwd_pack<E>(ed, dlo, dhi);
+      bwd_transposed_times_packed<D, E>(g_tr, 2 * h, plo, lane, acc_v);
+      bwd_transposed_times_packed<D, E>(g_tr, 2 * h + 1, phi, lane, acc_v);
+      bwd_transposed_times_packed<D, E>(q_tr, 2 * h, dlo, lane, acc_k);
+      bwd_transposed_times_packed<D, E>(q_tr, 2 * h + 1, dhi, lane, acc_k);
     }
   }
   if (active && l32 < nrows) {
