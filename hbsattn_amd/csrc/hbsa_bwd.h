@@ -117,21 +117,18 @@ __device__ __forceinline__ void bwd_stash_tile(const BwdTileRegs<D> &t, char *by
   }
 }
 
-// acc[h] (h = 0, 1: rows 0-31 / 32-63 of the tile) = tile rows . frag^T, the forward's S^T = K Q^T
+// rows 32*h .. 32*h+31 of the tile . frag^T, the forward's S^T = K Q^T for one half of a tile
 template <int D, typename E>
-__device__ __forceinline__ void bwd_rows_times_frag(const char *tile, const short8v *frag, int lane, f32x16 &a0, f32x16 &a1) {
+__device__ __forceinline__ f32x16 bwd_rows_times_frag(const char *tile, int h, const short8v *frag, int lane) {
   using T = BwdTile<D>;
   const int l32 = lane & 31, g32 = lane >> 5;
-  const int rd = l32 * T::RB + ((g32 ^ T::swz_rows(l32)) << 4);
+  const int rd = l32 * T::RB + ((g32 ^ T::swz_rows(l32)) << 4) + h * 32 * T::RB;
+  f32x16 a;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) { a0[i] = 0.f; a1[i] = 0.f; }
+  for (int i = 0; i < 16; ++i) a[i] = 0.f;
 #pragma unroll
-  for (int ks = 0; ks < T::KSTEPS; ++ks) {
-    const short8v x0 = *(const short8v *)(tile + (rd ^ (ks * 32)));
-    const short8v x1 = *(const short8v *)(tile + (rd ^ (ks * 32)) + 32 * T::RB);
-    a0 = E::mfma(x0, frag[ks], a0);
-    a1 = E::mfma(x1, frag[ks], a1);
-  }
+  for (int ks = 0; ks < T::KSTEPS; ++ks) a = E::mfma(*(const short8v *)(tile + (rd ^ (ks * 32))), frag[ks], a);
+  return a;
 }
 
 // acc[dt] += tile^T (rows 16*g .. 16*g+15 of the tile as the contraction index) . packed, the forward's
@@ -182,7 +179,7 @@ __device__ __forceinline__ void bwd_store_rows(char *row_ptr, const f32x16 *acc,
 
 // ---- dQ ----------------------------------------------------------------------------------------------
 template <int D, typename E>
-__global__ __launch_bounds__(kThreads, 1) void hbsa_bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   using T = BwdTile<D>;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   char *k_rows = lds, *k_tr = lds + T::TILE_BYTES, *v_rows = lds + 2 * T::TILE_BYTES;
@@ -263,20 +260,19 @@ __global__ __launch_bounds__(kThreads, 1) void hbsa_bwd_dq_kernel(BwdParams p) {
       bwd_fetch_tile<D>(vg + (int64_t)kpos * p.v_s, p.v_s, tile_valid(), vt);
     }
     if (!active) continue;
-    f32x16 s[2], dp[2];
-    bwd_rows_times_frag<D, E>(k_rows, qf, lane, s[0], s[1]);
-    bwd_rows_times_frag<D, E>(v_rows, dof, lane, dp[0], dp[1]);
     int lim = valid;   // keys of the tile below lim are visible to this lane's row
     if (p.causal) lim = min(lim, lane_kvis - cur_kpos + 1);
     lim -= 4 * g32;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
+      const f32x16 s = bwd_rows_times_frag<D, E>(k_rows, h, qf, lane);
+      const f32x16 dp = bwd_rows_times_frag<D, E>(v_rows, h, dof, lane);
       float e[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const bool vis = 32 * h + 8 * (i >> 2) + (i & 3) < lim;
-        const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[h][i], p.c, -lse2)) : 0.f;
-        e[i] = pv * (dp[h][i] - dlt);
+        const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], p.c, -lse2)) : 0.f;
+        e[i] = pv * (dp[i] - dlt);
       }
       short8v lo, hi;
       bwd_pack<E>(e, lo, hi);
@@ -393,15 +389,14 @@ __global__ __launch_bounds__(kThreads, 1) void hbsa_bwd_dkv_kernel(BwdParams p) 
     have = next_tile();
     if (have) fetch();   // on its way while this tile is computed on
     if (!active) continue;
-    f32x16 s[2], dp[2];
-    bwd_rows_times_frag<D, E>(q_rows, kf, lane, s[0], s[1]);
-    bwd_rows_times_frag<D, E>(g_rows, vf, lane, dp[0], dp[1]);
     // rows of the tile from first_vis on see this lane's key (causal); lanes past the block's keys see nothing
     int first_vis = 0;
     if (p.causal) first_vis = max(0, key_pos - shift - first_q_pos);
     if (l32 >= nrows) first_vis = 64;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
+      const f32x16 s = bwd_rows_times_frag<D, E>(q_rows, h, kf, lane);
+      const f32x16 dp = bwd_rows_times_frag<D, E>(g_rows, h, vf, lane);
       float ep[16], ed[16];
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
@@ -411,9 +406,9 @@ __global__ __launch_bounds__(kThreads, 1) void hbsa_bwd_dkv_kernel(BwdParams p) 
         for (int bq = 0; bq < 4; ++bq) {
           const int i = 4 * a + bq;
           const bool vis = rr0 + bq >= first_vis;   // rows past the block's end carry lse = +inf, hence P = 0
-          const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[h][i], p.c, -l4[bq])) : 0.f;
+          const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], p.c, -l4[bq])) : 0.f;
           ep[i] = pv;
-          ed[i] = pv * (dp[h][i] - d4[bq]);
+          ed[i] = pv * (dp[i] - d4[bq]);
         }
       }
       short8v plo, phi, dlo, dhi;
