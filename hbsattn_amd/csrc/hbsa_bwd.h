@@ -49,26 +49,28 @@ struct DeltaParams {
   int32_t total_q, nhead_q;
 };
 
-// delta[row, head] = sum over d of dO * O; one thread per (row, head)
+// delta[row, head] = sum over d of dO * O; D/8 neighbouring lanes share a (row, head), 16 bytes each
 template <int D, typename E>
 __global__ __launch_bounds__(256) void hbsa_bwd_delta_kernel(DeltaParams p) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= (int64_t)p.total_q * p.nhead_q) return;
-  const int64_t row = i / p.nhead_q;
-  const int h = (int)(i - row * p.nhead_q);
-  const char *o = p.out + row * p.o_s + h * p.o_h;
-  const char *g = p.dout + row * p.do_s + h * p.do_h;
+  constexpr int LPR = D / 8;   // lanes per row: 4, 8 or 16
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
+  const int ch = threadIdx.x % LPR;
+  const bool live = i < (int64_t)p.total_q * p.nhead_q;
   float acc = 0.f;
-#pragma unroll
-  for (int ch = 0; ch < D / 8; ++ch) {
-    const u32x4 a = *(const u32x4 *)(o + ch * 16), b = *(const u32x4 *)(g + ch * 16);
+  if (live) {
+    const int64_t row = i / p.nhead_q;
+    const int h = (int)(i - row * p.nhead_q);
+    const u32x4 a = *(const u32x4 *)(p.out + row * p.o_s + h * p.o_h + ch * 16);
+    const u32x4 b = *(const u32x4 *)(p.dout + row * p.do_s + h * p.do_h + ch * 16);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       acc += E::lo(a[j]) * E::lo(b[j]);
       acc += E::hi(a[j]) * E::hi(b[j]);
     }
   }
-  p.delta[i] = acc;
+#pragma unroll
+  for (int m = LPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m);
+  if (live && ch == 0) p.delta[i] = acc;
 }
 
 // ---- shared pieces of the two main kernels ---------------------------------------------------------
@@ -431,7 +433,7 @@ template <int D, typename E>
 int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_k_block, hipStream_t stream) {
   using T = BwdTile<D>;
   const int64_t rows = (int64_t)dp.total_q * dp.nhead_q;
-  hipLaunchKernelGGL((hbsa_bwd_delta_kernel<D, E>), dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream, dp);
+  hipLaunchKernelGGL((hbsa_bwd_delta_kernel<D, E>), dim3((unsigned)((rows * (D / 8) + 255) / 256)), dim3(256), 0, stream, dp);
   const int lds_dq = 3 * T::TILE_BYTES, lds_dkv = 4 * T::TILE_BYTES + 512;
   if (lds_dkv > 48 * 1024) {
     static thread_local bool raised[kMaxDevices] = {};
