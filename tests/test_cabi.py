@@ -94,6 +94,42 @@ def test_empty_problem_is_a_no_op():
     assert _lib.last_error() == ""
 
 
+def _call_bwd(lib, **over):
+    strides = (ctypes.c_int64 * 16)(*([4096, 128] * 8))
+    a = dict(q=256, k=256, v=256, out=256, dout=256, lse=256, dq=256, dk=256, dv=256, cu_k=256, cu_nqb=256, cu_nkb=256,
+             ws=256, ws_bytes=1 << 30, bws=256, bws_bytes=1 << 30, dtype=0, batch=1, total_q=128, total_k=128, hq=32, hk=32,
+             d=128, nqb=1, nkb=1, qbs=128, kbs=128, causal=1, scale=0.1)
+    a.update(over)
+    return lib.hbsa_bwd(a["q"], a["k"], a["v"], a["out"], a["dout"], a["lse"], a["dq"], a["dk"], a["dv"], a["cu_k"],
+                        a["cu_nqb"], a["cu_nkb"], a["ws"], a["ws_bytes"], a["bws"], a["bws_bytes"], a["dtype"], a["batch"],
+                        a["total_q"], a["total_k"], a["hq"], a["hk"], a["d"], a["nqb"], a["nkb"], a["qbs"], a["kbs"],
+                        a["causal"], a["scale"], strides, None)
+
+
+@pytest.mark.parametrize("over,code,needle", [
+    (dict(dout=None), -1, "null"),
+    (dict(dtype=2), -2, "bf16 or fp16"),
+    (dict(d=96), -2, "headdim"),
+    (dict(kbs=40), -1, "multiples of 16"),
+    (dict(dq=264), -1, "aligned"),
+    (dict(ws_bytes=16), -3, "workspace"),
+    (dict(bws_bytes=16), -3, "bwd_workspace"),
+])
+def test_backward_argument_validation_without_touching_the_gpu(over, code, needle):
+    lib = _lib.load()
+    rc = _call_bwd(lib, **over)
+    assert rc == code
+    assert needle in _lib.last_error()
+
+
+def test_backward_workspace_bytes_and_empty_problem():
+    lib = _lib.load()
+    assert lib.hbsa_bwd_workspace_bytes(100, 8) == 3328      # 100 * 8 floats, rounded up to 256 bytes
+    assert lib.hbsa_bwd_workspace_bytes(0, 8) == 0
+    assert _call_bwd(lib, total_q=0) == 0
+    assert _lib.last_error() == ""
+
+
 def _c_calculate_blocks(cu, block_size):
     import numpy as np
     lib = _lib.load()
