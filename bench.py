@@ -127,6 +127,23 @@ def measure(name, steps, warmup):
     return w, res
 
 
+def measure_backward(w, flops, steps):
+    """Device time of one backward call (delta, dq and dk/dv kernels) for the workload's tensors, with
+    event pairs on the launch stream; FLOPs counted as 2.5 x the forward's over kept blocks."""
+    from hbsattn_amd.interface import hbsa_backward, hbsa_prepare, hbsa_run
+
+    prepared = hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, w.q_block_size, w.k_block_size, w.causal,
+                            w.q_meta[0], w.q_meta[2], w.q_meta[3], w.k_meta[0], w.k_meta[3])
+    out, lse = hbsa_run(w.q, w.k, w.v, prepared, w.softmax_scale, return_lse=True)
+    dout = torch.randn(out.shape, dtype=torch.float32, device=out.device, generator=torch.Generator(out.device).manual_seed(5)).to(out.dtype)
+    step = lambda: hbsa_backward(w.q, w.k, w.v, out, dout, lse, prepared, w.softmax_scale)
+    for _ in range(min(3, steps)):
+        step()
+    ms = time_kernel_events(step, steps)
+    return {"ms_per_call": ms, "tflops": 2.5 * flops / ms / 1e9, "flops_counted": "2.5 x forward FLOPs over kept blocks",
+            "kernels": "hbsa_bwd_delta_kernel + hbsa_bwd_dq_kernel + hbsa_bwd_dkv_kernel"}
+
+
 def cpu_baseline(w, budget_s=20.0):
     """The CPU oracle on (sequence, kv head) pairs of the workload, in sequence-major order, one
     pair at a time until the budget is spent; throughput in the metric's unit from the sample's own
@@ -180,6 +197,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-target", action="store_true", help="skip the extra measurement at the 32K target shape")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--backward", action="store_true", help="also time the backward kernels (reported under 'backward')")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a 1 GiB device-to-device copy K times (the known-size kernel the HBM counters "
                          "of a profile are scaled by)")
@@ -219,6 +237,8 @@ def main():
         "detail": {k: res[k] for k in ("per_call_sync_ms", "attention_kernel_ms", "prepass_ms", "tflops_exact_elements",
                                        "flops", "bytes", "visited_pairs")},
     }
+    if a.backward:
+        line["backward"] = measure_backward(w, res["flops"], max(1, a.steps // 5))
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, a.cpu_budget)
     del w

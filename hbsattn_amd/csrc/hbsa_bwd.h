@@ -288,7 +288,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
 
 // ---- dK, dV ------------------------------------------------------------------------------------------
 template <int D, typename E>
-__global__ __launch_bounds__(kThreads, 1) void hbsa_bwd_dkv_kernel(BwdParams p) {
+__global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel(BwdParams p) {
   using T = BwdTile<D>;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   char *q_rows = lds, *q_tr = lds + T::TILE_BYTES, *g_rows = lds + 2 * T::TILE_BYTES, *g_tr = lds + 3 * T::TILE_BYTES;
