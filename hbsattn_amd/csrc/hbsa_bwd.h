@@ -395,10 +395,27 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
     int first_vis = 0;
     if (p.causal) first_vis = max(0, key_pos - shift - first_q_pos);
     if (l32 >= nrows) first_vis = 64;
+    // With one workgroup per CU (D = 128) registers are plentiful: both halves' S and dP are formed
+    // first, so that the matrix products of one half can overlap the vector work of the other.
+    constexpr bool kEager = D > 64;
+    f32x16 s2[2], dp2[2];
+    if constexpr (kEager) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        s2[h] = bwd_rows_times_frag<D, E>(q_rows, h, kf, lane);
+        dp2[h] = bwd_rows_times_frag<D, E>(g_rows, h, vf, lane);
+      }
+    }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const f32x16 s = bwd_rows_times_frag<D, E>(q_rows, h, kf, lane);
-      const f32x16 dp = bwd_rows_times_frag<D, E>(g_rows, h, vf, lane);
+      f32x16 s, dp;
+      if constexpr (kEager) {
+        s = s2[h];
+        dp = dp2[h];
+      } else {
+        s = bwd_rows_times_frag<D, E>(q_rows, h, kf, lane);
+        dp = bwd_rows_times_frag<D, E>(g_rows, h, vf, lane);
+      }
       float ep[16], ed[16];
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
