@@ -446,20 +446,217 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
   }
 }
 
+// ---- dK, dV at D = 128: eight wavefronts -------------------------------------------------------------
+// The kernel above holds K^T, V^T and both accumulators of a wavefront in registers: 256 + 238 at
+// D = 128, one wavefront per SIMD.  This one keeps the workgroup's K and V rows in LDS (read as B
+// operands per product) and runs eight wavefronts: wavefronts w and w + 4 own the same 32 keys and
+// take rows 0-31 and 32-63 of every tile, so that two wavefronts share a SIMD and cover each other's
+// waits; their two partial accumulators are added through LDS at the end.  No product is computed twice.
+template <typename E>
+__global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
+  constexpr int D = 128;
+  using T = BwdTile<D>;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  char *q_rows = lds, *q_tr = lds + T::TILE_BYTES, *g_rows = lds + 2 * T::TILE_BYTES, *g_tr = lds + 3 * T::TILE_BYTES;
+  float *lse_s = (float *)(lds + 4 * T::TILE_BYTES);   // [64] log2-domain log-sum-exp of the tile's rows
+  float *dlt_s = lse_s + 64;                           // [64] their delta
+  char *k_blk = lds + 4 * T::TILE_BYTES + 512;         // [128][D] keys of the workgroup, layout read by rows
+  char *v_blk = k_blk + 2 * T::TILE_BYTES;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int slot = wave & 3, half = wave >> 2;   // 32-key slot of the workgroup; which 32 rows of a tile
+  const int g32 = lane >> 5, l32 = lane & 31;
+  const int hk = blockIdx.y;
+  const int kb = blockIdx.x / p.nsub_k, sub = blockIdx.x - kb * p.nsub_k;
+
+  int b = 0;   // the sequence the k block belongs to
+  while (b + 1 < p.batch && p.cu_num_k_block[b + 1] <= kb) ++b;
+  const int kbl = kb - p.cu_num_k_block[b];
+  const int k0 = p.cu_k[b], klen = p.cu_k[b + 1] - k0;
+  const int krows = min(p.kbs, klen - kbl * p.kbs);
+  const int wg_row0 = sub * 4 * kWaveRows;                 // first key of the workgroup inside the block
+  const int row0 = wg_row0 + slot * kWaveRows;
+  const int nrows = min(kWaveRows, krows - row0);
+  const bool active = nrows > 0;
+  const int key_pos = kbl * p.kbs + min(row0 + l32, krows - 1);
+  const int wg_first_key = kbl * p.kbs + wg_row0;
+
+  // the workgroup's 128 key rows (rows past the block's end repeat its last key; their lanes are masked)
+  {
+    const char *kbase = p.k + (int64_t)(k0 + kbl * p.kbs) * p.k_s + (int64_t)hk * p.k_h;
+    const char *vbase = p.v + (int64_t)(k0 + kbl * p.kbs) * p.v_s + (int64_t)hk * p.v_h;
+#pragma unroll
+    for (int i = 0; i < 128 * T::CPR / 512; ++i) {
+      const int ch = i * 512 + threadIdx.x;
+      const int r = ch / T::CPR, pc = ch % T::CPR;
+      const int64_t src_row = min(wg_row0 + r, krows - 1);
+      const int dst = r * T::RB + ((pc ^ T::swz_rows(r)) << 4);
+      *(u32x4 *)(k_blk + dst) = *(const u32x4 *)(kbase + src_row * p.k_s + pc * 16);
+      *(u32x4 *)(v_blk + dst) = *(const u32x4 *)(vbase + src_row * p.v_s + pc * 16);
+    }
+  }
+  f32x16 acc_k[T::DT], acc_v[T::DT];
+#pragma unroll
+  for (int dt = 0; dt < T::DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { acc_k[dt][i] = 0.f; acc_v[dt][i] = 0.f; }
+
+  int qb = p.cu_num_q_block[b] - 1, r = 0, qoff = 0;
+  const int qb_end = p.cu_num_q_block[b + 1];
+  QBlockInfo inf = {};
+  auto tile_reaches = [&]() {
+    return !p.causal || inf.q_pos + qoff + min(64, inf.rows - qoff) - 1 + inf.shift >= wg_first_key;
+  };
+  auto next_tile = [&]() -> bool {
+    for (;;) {
+      if (qb >= p.cu_num_q_block[b]) {
+        qoff += 64;
+        if (qoff >= inf.rows) { qoff = 0; ++r; }
+        if (r < p.ratio) {
+          if (tile_reaches()) return true;
+          continue;
+        }
+      }
+      for (++qb; qb < qb_end; ++qb) {
+        const uint32_t word = p.bits[((size_t)hk * p.nqb + qb) * p.wpr + (kbl >> 5)];
+        if ((word >> (kbl & 31)) & 1u) break;
+      }
+      if (qb >= qb_end) return false;
+      inf = p.info[qb];
+      r = 0;
+      qoff = -64;
+    }
+  };
+  // a tile's chunks over 512 threads: two per thread and tensor
+  u32x4 qt[2], gt[2];
+  float l2_next = INFINITY, dl_next = 0.f;
+  auto fetch = [&]() {
+    const int valid = min(64, inf.rows - qoff);
+    const int64_t row_first = inf.row_begin + qoff;
+    const int hq = hk * p.ratio + r;
+    const char *qsrc = p.q + row_first * p.q_s + (int64_t)hq * p.q_h;
+    const char *gsrc = p.dout + row_first * p.do_s + (int64_t)hq * p.do_h;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int ch = i * 512 + threadIdx.x;
+      const int rr = min(ch / T::CPR, valid - 1), pc = ch % T::CPR;
+      qt[i] = *(const u32x4 *)(qsrc + (int64_t)rr * p.q_s + pc * 16);
+      gt[i] = *(const u32x4 *)(gsrc + (int64_t)rr * p.do_s + pc * 16);
+    }
+    l2_next = INFINITY;
+    dl_next = 0.f;
+    if (threadIdx.x < valid) {
+      const float l = p.lse[(row_first + threadIdx.x) * p.nhead_q + hq];
+      l2_next = l == -INFINITY ? INFINITY : l * kLog2e;
+      dl_next = p.delta[(row_first + threadIdx.x) * p.nhead_q + hq];
+    }
+  };
+  const int rd = l32 * T::RB + ((g32 ^ T::swz_rows(l32)) << 4);   // this lane's 16 bytes of row l32, k-step 0
+  bool have = next_tile();
+  if (have) fetch();
+  while (have) {
+    const int first_q_pos = inf.q_pos + qoff, shift = inf.shift;
+    __syncthreads();   // the previous tile has been read by every wavefront (and, the first time, K and V are in place)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int ch = i * 512 + threadIdx.x;
+      const int rr = ch / T::CPR, pc = ch % T::CPR;
+      const int by_rows = rr * T::RB + ((pc ^ T::swz_rows(rr)) << 4), tr = rr * T::RB + ((pc ^ T::swz_tr(rr)) << 4);
+      *(u32x4 *)(q_rows + by_rows) = qt[i];
+      *(u32x4 *)(q_tr + tr) = qt[i];
+      *(u32x4 *)(g_rows + by_rows) = gt[i];
+      *(u32x4 *)(g_tr + tr) = gt[i];
+    }
+    if (threadIdx.x < 64) {
+      lse_s[threadIdx.x] = l2_next;
+      dlt_s[threadIdx.x] = dl_next;
+    }
+    __syncthreads();
+    have = next_tile();
+    if (have) fetch();
+    if (!active) continue;
+    int first_vis = 0;
+    if (p.causal) first_vis = max(0, key_pos - shift - first_q_pos);
+    if (l32 >= nrows) first_vis = 64;
+    // rows 32*half .. +31 of the tile against this wavefront's 32 keys
+    f32x16 sv, dp;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { sv[i] = 0.f; dp[i] = 0.f; }
+#pragma unroll
+    for (int ks = 0; ks < T::KSTEPS; ++ks) {
+      const int a_off = (rd ^ (ks * 32)) + half * 32 * T::RB, b_off = (rd ^ (ks * 32)) + slot * 32 * T::RB;
+      sv = E::mfma(*(const short8v *)(q_rows + a_off), *(const short8v *)(k_blk + b_off), sv);
+      dp = E::mfma(*(const short8v *)(g_rows + a_off), *(const short8v *)(v_blk + b_off), dp);
+    }
+    float ep[16], ed[16];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int rr0 = 32 * half + 8 * a + 4 * g32;
+      const f32x4 l4 = *(const f32x4 *)(lse_s + rr0), d4 = *(const f32x4 *)(dlt_s + rr0);
+#pragma unroll
+      for (int bq = 0; bq < 4; ++bq) {
+        const int i = 4 * a + bq;
+        const bool vis = rr0 + bq >= first_vis;   // rows past the block's end carry lse = +inf, hence P = 0
+        const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(sv[i], p.c, -l4[bq])) : 0.f;
+        ep[i] = pv;
+        ed[i] = pv * (dp[i] - d4[bq]);
+      }
+    }
+    short8v plo, phi, dlo, dhi;
+    bwd_pack<E>(ep, plo, phi);
+    bwd_pack<E>(ed, dlo, dhi);
+    bwd_transposed_times_packed<D, E>(g_tr, 2 * half, plo, lane, acc_v);
+    bwd_transposed_times_packed<D, E>(g_tr, 2 * half + 1, phi, lane, acc_v);
+    bwd_transposed_times_packed<D, E>(q_tr, 2 * half, dlo, lane, acc_k);
+    bwd_transposed_times_packed<D, E>(q_tr, 2 * half + 1, dhi, lane, acc_k);
+  }
+  // wavefronts 4-7 hand their partial sums to wavefronts 0-3 through LDS: [slot][register][lane] floats
+  __syncthreads();
+  float *xch = (float *)lds + (size_t)slot * 128 * 64 + lane;
+  if (half == 1) {
+#pragma unroll
+    for (int dt = 0; dt < T::DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        xch[(dt * 16 + i) * 64] = acc_k[dt][i];
+        xch[(64 + dt * 16 + i) * 64] = acc_v[dt][i];
+      }
+  }
+  __syncthreads();
+  if (half == 0 && active) {
+#pragma unroll
+    for (int dt = 0; dt < T::DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        acc_k[dt][i] += xch[(dt * 16 + i) * 64];
+        acc_v[dt][i] += xch[(64 + dt * 16 + i) * 64];
+      }
+    if (l32 < nrows) {
+      const int64_t row = k0 + kbl * p.kbs + row0 + l32;
+      bwd_store_rows<D, E>(p.dk + row * p.dk_s + (int64_t)hk * p.dk_h, acc_k, p.scale, g32);
+      bwd_store_rows<D, E>(p.dv + row * p.dv_s + (int64_t)hk * p.dv_h, acc_v, 1.f, g32);
+    }
+  }
+}
+
 template <int D, typename E>
 int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_k_block, hipStream_t stream) {
   using T = BwdTile<D>;
   const int64_t rows = (int64_t)dp.total_q * dp.nhead_q;
   hipLaunchKernelGGL((hbsa_bwd_delta_kernel<D, E>), dim3((unsigned)((rows * (D / 8) + 255) / 256)), dim3(256), 0, stream, dp);
-  const int lds_dq = 3 * T::TILE_BYTES, lds_dkv = 4 * T::TILE_BYTES + 512;
+  // D = 128: tiles, the rows' lse and delta, K and V of the workgroup; at least the 128 KB of the final exchange
+  const int lds_dq = 3 * T::TILE_BYTES, lds_dkv = D == 128 ? 8 * T::TILE_BYTES + 512 : 4 * T::TILE_BYTES + 512;
   if (lds_dkv > 48 * 1024) {
     static thread_local bool raised[kMaxDevices] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
       return fail(HBSA_ERR_UNSUPPORTED, "no current device, or device index above %d", kMaxDevices - 1);
     if (!raised[dev]) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&hbsa_bwd_dkv_kernel<D, E>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv);
+      const void *dkv = nullptr;
+      if constexpr (D == 128) dkv = reinterpret_cast<const void *>(&hbsa_bwd_dkv8_kernel<E>);
+      else dkv = reinterpret_cast<const void *>(&hbsa_bwd_dkv_kernel<D, E>);
+      hipError_t e = hipFuncSetAttribute(dkv, hipFuncAttributeMaxDynamicSharedMemorySize, lds_dkv);
       if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(&hbsa_bwd_dq_kernel<D, E>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds_dq);
@@ -469,8 +666,13 @@ int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_
   }
   hipLaunchKernelGGL((hbsa_bwd_dq_kernel<D, E>), dim3((unsigned)(bp.nqb * bp.nsub), (unsigned)nhead_k), dim3(kThreads), lds_dq,
                      stream, bp);
-  hipLaunchKernelGGL((hbsa_bwd_dkv_kernel<D, E>), dim3((unsigned)(num_k_block * bp.nsub_k), (unsigned)nhead_k), dim3(kThreads),
-                     lds_dkv, stream, bp);
+  if constexpr (D == 128) {
+    hipLaunchKernelGGL((hbsa_bwd_dkv8_kernel<E>), dim3((unsigned)(num_k_block * bp.nsub_k), (unsigned)nhead_k), dim3(512),
+                       lds_dkv, stream, bp);
+  } else {
+    hipLaunchKernelGGL((hbsa_bwd_dkv_kernel<D, E>), dim3((unsigned)(num_k_block * bp.nsub_k), (unsigned)nhead_k),
+                       dim3(kThreads), lds_dkv, stream, bp);
+  }
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
 }
