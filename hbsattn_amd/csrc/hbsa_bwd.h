@@ -15,7 +15,8 @@
 //                           Per 64-key tile  S^T = K Q^T,  dP^T = V dO^T  (A = tile rows from LDS,
 //                           B = Q^T / dO^T in registers),  dS^T in the accumulator layout is the B
 //                           operand of  dQ^T += K^T dS^T  (A = K^T through transposing LDS reads).
-//   hbsa_bwd_dkv_kernel   : (head dims up to 64; D = 128 has its own form below) the same with the roles of queries and keys exchanged: one workgroup per
+//   hbsa_bwd_dkv_kernel   : (head dims up to 64; hbsa_bwd_dkv8_kernel is the form for D = 128) the same
+//                           with the roles of queries and keys exchanged: one workgroup per
 //                           (kv head, k block, group of four 32-key slots); K^T and V^T stay in
 //                           registers, the Q and dO rows of every q block that keeps the k block (and of
 //                           every q head of the group) stream through LDS in 64-row tiles:
