@@ -191,7 +191,9 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g32 = lane >> 5, l32 = lane & 31;
   const int hk = blockIdx.y;
-  const int qb = blockIdx.x / p.nsub, sub = blockIdx.x - qb * p.nsub;
+  // last q blocks first: under a causal mask they are the long ones, and the grid should not end on them
+  const int qb_rev = blockIdx.x / p.nsub, sub = blockIdx.x - qb_rev * p.nsub;
+  const int qb = p.nqb - 1 - qb_rev;
   const QBlockInfo inf = p.info[qb];
 
   const int slot = sub * 4 + wave;
