@@ -210,30 +210,35 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = 
 
 
 def backward_supported(q: torch.Tensor) -> bool:
-    """The backward kernels take bf16 / fp16 tensors with a native head dim (32, 64 or 128)."""
-    return q.dtype in (torch.bfloat16, torch.float16) and q.dim() == 3 and q.shape[2] in _NATIVE_HEADDIMS
+    """The backward kernels take bf16 / fp16 tensors; head dims up to 128 (others than 32, 64, 128 run
+    zero-padded, like the forward)."""
+    return q.dtype in (torch.bfloat16, torch.float16) and q.dim() == 3 and 0 < q.shape[2] <= _NATIVE_HEADDIMS[-1]
 
 
 def hbsa_backward(q, k, v, out, dout, lse, prepared: PreparedMask, softmax_scale):
     """``(dq, dk, dv)`` through ``hbsa_bwd`` on the current stream.  ``out`` and ``lse`` are what
     ``hbsa_run(..., return_lse=True)`` returned for the same q, k, v, prepared mask and scale."""
     if not backward_supported(q):
-        raise NotImplementedError("hbsattn_amd: the backward takes bfloat16 / float16 tensors with headdim 32, 64 or 128")
+        raise NotImplementedError("hbsattn_amd: the backward takes bfloat16 / float16 tensors with headdim <= 128")
     if prepared.cu_k_seqlens is None:
         raise ValueError("this PreparedMask was built without the sequence boundaries the backward needs")
     lib = _lib.load()
     total_q, nhead_q, headdim = q.shape
     total_k, nhead_k = k.shape[0], k.shape[1]
     scale = float(softmax_scale) if softmax_scale is not None else headdim ** -0.5
-    q = q if _rows_ok(q) else q.contiguous()
-    k = k if _rows_ok(k) else k.contiguous()
-    v = v if _rows_ok(v) else v.contiguous()
-    out = out if _rows_ok(out) else out.contiguous()
-    dout = dout if _rows_ok(dout) else dout.contiguous()
+    if total_q == 0 or total_k == 0:
+        return torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    d_run = next(d for d in _NATIVE_HEADDIMS if d >= headdim)
+    if d_run != headdim:  # zero columns change neither q.k nor rowsum(dout * out) and get zero gradients
+        q, k, v, out, dout = (_pad_headdim(t, d_run) for t in (q, k, v, out, dout))
+    else:
+        q = q if _rows_ok(q) else q.contiguous()
+        k = k if _rows_ok(k) else k.contiguous()
+        v = v if _rows_ok(v) else v.contiguous()
+        out = out if _rows_ok(out) else out.contiguous()
+        dout = dout if _rows_ok(dout) else dout.contiguous()
     lse = lse.contiguous()
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    if total_q == 0 or total_k == 0:
-        return dq.zero_(), dk.zero_(), dv.zero_()
     bws_bytes = int(lib.hbsa_bwd_workspace_bytes(total_q, nhead_q))
     bws = torch.empty(bws_bytes, dtype=torch.uint8, device=q.device)
     strides = (ctypes.c_int64 * 16)(q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
@@ -245,11 +250,13 @@ def hbsa_backward(q, k, v, out, dout, lse, prepared: PreparedMask, softmax_scale
                           dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), prepared.cu_k_seqlens.data_ptr(),
                           prepared.cu_num_q_block.data_ptr(), prepared.cu_num_k_block.data_ptr(), ws.data_ptr(), ws.numel(),
                           bws.data_ptr(), bws_bytes, _dtype_code(q.dtype), prepared.cu_k_seqlens.numel() - 1, total_q,
-                          total_k, nhead_q, nhead_k, headdim, prepared.num_q_block, prepared.num_k_block,
+                          total_k, nhead_q, nhead_k, d_run, prepared.num_q_block, prepared.num_k_block,
                           prepared.q_block_size, prepared.k_block_size, int(prepared.causal), scale, strides,
                           torch.cuda.current_stream().cuda_stream)
     if rc != 0:
         raise RuntimeError(f"hbsa_bwd failed (code {rc}): {_lib.last_error()}")
+    if d_run != headdim:
+        dq, dk, dv = (t[:, :, :headdim].contiguous() for t in (dq, dk, dv))
     return dq, dk, dv
 
 

@@ -81,6 +81,18 @@ def test_gradients_match_oracle(case, dtype):
     _check(dv, rdv, "dv")
 
 
+@pytest.mark.parametrize("d", [16, 18, 40, 96])
+def test_head_dims_that_run_zero_padded(d):
+    q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(20 + d, [90, 33], [70, 120], 4, 2, d, 32, 32, 0.6, torch.bfloat16)
+    print(f"backward padded head dim {d}", flush=True)
+    _, dq, dk, dv = _gpu_grads(q, k, v, do, cq, ck, mask, 32, 32, True, None)
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    rdq, rdk, rdv = hbsa_oracle_grads(q, k, v, do, cu_q, cu_k, mask, 32, 32, True, None)
+    _check(dq, rdq, "dq")
+    _check(dk, rdk, "dk")
+    _check(dv, rdv, "dv")
+
+
 def test_rows_without_visible_keys_and_unkept_keys_get_exact_zeros():
     # q longer than k under bottom-right causal alignment: the first 32 rows see no key; k block 1 is kept by nobody
     q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(11, [48], [32], 2, 1, 32, 16, 16, 1.1, torch.bfloat16)
