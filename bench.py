@@ -141,7 +141,7 @@ def measure_backward(w, flops, steps):
         step()
     ms = time_kernel_events(step, steps)
     return {"ms_per_call": ms, "tflops": 2.5 * flops / ms / 1e9, "flops_counted": "2.5 x forward FLOPs over kept blocks",
-            "kernels": "hbsa_bwd_delta_kernel + hbsa_bwd_dq_kernel + hbsa_bwd_dkv_kernel"}
+            "kernels": "hbsa_bwd_delta_kernel + hbsa_bwd_dq_kernel + hbsa_bwd_dkv8_kernel (hbsa_bwd_dkv_kernel below D=128)"}
 
 
 def cpu_baseline(w, budget_s=20.0):
