@@ -15,6 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _ROOT = os.path.dirname(_HERE)
 SOURCES = [os.path.join(_HERE, "csrc", "hbsa_fwd.hip")]
 OUTPUT = os.path.join(_HERE, "libhbsattn_amd.so")
+HAND_ISSUED_READS = "hbsa_fwd_kernel"   # substring of the mangled names of the kernels with hand-issued LDS reads
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
 HIPCC_FLAGS = [
@@ -44,14 +45,18 @@ def build(verbose: bool = False) -> str:
     if res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
         raise RuntimeError("hipcc failed: " + " ".join(cmd))
-    # The attention kernels issue their LDS reads by hand and wait for them by count.  The compiler
-    # does not know that such a register has a read in flight; if it spills one, it saves the
-    # register before the data has arrived and the result is wrong now and then.  So a build in
-    # which any kernel spills vector registers is refused.
+    # The forward attention kernel issues its LDS reads by hand and waits for them by count.  The
+    # compiler does not know that such a register has a read in flight; if it spills one, it saves the
+    # register before the data has arrived and the result is wrong now and then.  So a build in which
+    # that kernel spills vector registers is refused.  (The other kernels leave every wait to the
+    # compiler; a spill there only costs time and is reported.)
     spills = _vgpr_spills(res.stderr)
-    if spills:
+    fatal = {k: v for k, v in spills.items() if HAND_ISSUED_READS in k}
+    if fatal:
         os.remove(OUTPUT)
-        raise RuntimeError(f"vector-register spills in {spills}: reduce register pressure (see the comment here)")
+        raise RuntimeError(f"vector-register spills in {fatal}: reduce register pressure (see the comment here)")
+    if spills and verbose:
+        print(f"note: vector-register spills in {spills}")
     if verbose:
         print(" ".join(cmd))
     return OUTPUT

@@ -234,17 +234,22 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
 
   // the tile sequence: 64-key tiles of the kept k blocks, cut at the last key any row of the block sees
   int j = -1, kpos = 0;
+  int word_base = -32;      // k block of bit 0 of the word being walked
+  uint32_t word_left = 0;   // its kept blocks not visited yet
   auto next_tile = [&]() -> bool {
     if (j >= 0) {
       kpos += kTileKeys;
       if (kpos < min((j + 1) * p.kbs, inf.kmax)) return true;
     }
-    for (++j; j < inf.nkblk; ++j)
-      if ((bits[j >> 5] >> (j & 31)) & 1u) {
-        kpos = j * p.kbs;   // below kmax: the pre-pass cleared the bits of blocks no row can see
-        return true;
-      }
-    return false;
+    while (word_left == 0) {   // one load per 32 k blocks, kept or not
+      word_base += 32;
+      if (word_base >= inf.nkblk) return false;
+      word_left = bits[word_base >> 5];
+    }
+    j = word_base + __builtin_ctz(word_left);
+    word_left &= word_left - 1;
+    kpos = j * p.kbs;   // below kmax: the pre-pass cleared the bits of blocks no row can see
+    return true;
   };
   auto tile_valid = [&]() { return min(kTileKeys, min((j + 1) * p.kbs, inf.kmax) - kpos); };
   BwdTileRegs<D> kt, vt;
@@ -339,6 +344,8 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
   // key of this workgroup)
   int qb = p.cu_num_q_block[b] - 1, r = 0, qoff = 0;
   const int qb_end = p.cu_num_q_block[b + 1];
+  int kept_base = p.cu_num_q_block[b] - 64;   // q blocks kept_base .. +63: those that keep this k block, not visited yet
+  uint64_t kept = 0;
   QBlockInfo inf = {};
   auto tile_reaches = [&]() {
     return !p.causal || inf.q_pos + qoff + min(64, inf.rows - qoff) - 1 + inf.shift >= wg_first_key;
@@ -353,11 +360,15 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
           continue;
         }
       }
-      for (++qb; qb < qb_end; ++qb) {
-        const uint32_t word = p.bits[((size_t)hk * p.nqb + qb) * p.wpr + (kbl >> 5)];
-        if ((word >> (kbl & 31)) & 1u) break;
+      while (kept == 0) {   // one load per 64 q blocks: lane i looks at q block kept_base + i
+        kept_base += 64;
+        if (kept_base >= qb_end) return false;
+        uint32_t word = 0;
+        if (kept_base + lane < qb_end) word = p.bits[((size_t)hk * p.nqb + kept_base + lane) * p.wpr + (kbl >> 5)];
+        kept = __ballot((word >> (kbl & 31)) & 1u);
       }
-      if (qb >= qb_end) return false;
+      qb = kept_base + __builtin_ctzll(kept);
+      kept &= kept - 1;
       inf = p.info[qb];
       r = 0;
       qoff = -64;   // the step above moves to the block's first tile
@@ -507,6 +518,8 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
 
   int qb = p.cu_num_q_block[b] - 1, r = 0, qoff = 0;
   const int qb_end = p.cu_num_q_block[b + 1];
+  int kept_base = p.cu_num_q_block[b] - 64;   // q blocks kept_base .. +63: those that keep this k block, not visited yet
+  uint64_t kept = 0;
   QBlockInfo inf = {};
   auto tile_reaches = [&]() {
     return !p.causal || inf.q_pos + qoff + min(64, inf.rows - qoff) - 1 + inf.shift >= wg_first_key;
@@ -521,11 +534,15 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
           continue;
         }
       }
-      for (++qb; qb < qb_end; ++qb) {
-        const uint32_t word = p.bits[((size_t)hk * p.nqb + qb) * p.wpr + (kbl >> 5)];
-        if ((word >> (kbl & 31)) & 1u) break;
+      while (kept == 0) {   // one load per 64 q blocks: lane i looks at q block kept_base + i
+        kept_base += 64;
+        if (kept_base >= qb_end) return false;
+        uint32_t word = 0;
+        if (kept_base + lane < qb_end) word = p.bits[((size_t)hk * p.nqb + kept_base + lane) * p.wpr + (kbl >> 5)];
+        kept = __ballot((word >> (kbl & 31)) & 1u);
       }
-      if (qb >= qb_end) return false;
+      qb = kept_base + __builtin_ctzll(kept);
+      kept &= kept - 1;
       inf = p.info[qb];
       r = 0;
       qoff = -64;
