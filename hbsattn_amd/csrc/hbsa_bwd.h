@@ -36,7 +36,7 @@ struct BwdParams {
   const uint32_t *bits;
   const int32_t *cu_k, *cu_num_q_block, *cu_num_k_block;
   int64_t q_s, q_h, k_s, k_h, v_s, v_h, do_s, do_h, dq_s, dq_h, dk_s, dk_h, dv_s, dv_h;   // bytes
-  int32_t nqb, batch, ratio, nhead_q, kbs, wpr, causal;
+  int32_t nqb, batch, ratio, nhead_q, qbs, kbs, wpr, causal;
   int32_t wps, nsub;     // q side: wave slots per q head and workgroups per (kv head, q block), as in the forward
   int32_t nsub_k;        // k side: workgroups per (kv head, k block) = ceil(k_block_size / 128)
   float c;               // softmax_scale * log2(e), signed
@@ -344,15 +344,23 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
   // key of this workgroup)
   int qb = p.cu_num_q_block[b] - 1, r = 0, qoff = 0;
   const int qb_end = p.cu_num_q_block[b + 1];
-  int kept_base = p.cu_num_q_block[b] - 64;   // q blocks kept_base .. +63: those that keep this k block, not visited yet
+  const int qb_begin = p.cu_num_q_block[b];
+  int kept_base = qb_begin - 64;   // q blocks kept_base .. +63: those that keep this k block, not visited yet
   uint64_t kept = 0;
   QBlockInfo inf = {};
+  int seq_row0 = 0, seq_qlen = 0;   // first query row and query count of the sequence
+  if (qb_begin < qb_end) {
+    const QBlockInfo first = p.info[qb_begin];
+    seq_row0 = first.row_begin;
+    seq_qlen = klen - first.shift;
+    inf.shift = first.shift;
+  }
   auto tile_reaches = [&]() {
     return !p.causal || inf.q_pos + qoff + min(64, inf.rows - qoff) - 1 + inf.shift >= wg_first_key;
   };
   auto next_tile = [&]() -> bool {
     for (;;) {
-      if (qb >= p.cu_num_q_block[b]) {   // inside a kept q block: next tile, then next head
+      if (qb >= qb_begin) {   // inside a kept q block: next tile, then next head
         qoff += 64;
         if (qoff >= inf.rows) { qoff = 0; ++r; }
         if (r < p.ratio) {
@@ -369,7 +377,10 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
       }
       qb = kept_base + __builtin_ctzll(kept);
       kept &= kept - 1;
-      inf = p.info[qb];
+      // the q block's geometry follows from the sequence's (no load on this path)
+      inf.q_pos = (qb - qb_begin) * p.qbs;
+      inf.row_begin = seq_row0 + inf.q_pos;
+      inf.rows = min(p.qbs, seq_qlen - inf.q_pos);
       r = 0;
       qoff = -64;   // the step above moves to the block's first tile
     }
@@ -518,15 +529,23 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
 
   int qb = p.cu_num_q_block[b] - 1, r = 0, qoff = 0;
   const int qb_end = p.cu_num_q_block[b + 1];
-  int kept_base = p.cu_num_q_block[b] - 64;   // q blocks kept_base .. +63: those that keep this k block, not visited yet
+  const int qb_begin = p.cu_num_q_block[b];
+  int kept_base = qb_begin - 64;   // q blocks kept_base .. +63: those that keep this k block, not visited yet
   uint64_t kept = 0;
   QBlockInfo inf = {};
+  int seq_row0 = 0, seq_qlen = 0;   // first query row and query count of the sequence
+  if (qb_begin < qb_end) {
+    const QBlockInfo first = p.info[qb_begin];
+    seq_row0 = first.row_begin;
+    seq_qlen = klen - first.shift;
+    inf.shift = first.shift;
+  }
   auto tile_reaches = [&]() {
     return !p.causal || inf.q_pos + qoff + min(64, inf.rows - qoff) - 1 + inf.shift >= wg_first_key;
   };
   auto next_tile = [&]() -> bool {
     for (;;) {
-      if (qb >= p.cu_num_q_block[b]) {
+      if (qb >= qb_begin) {
         qoff += 64;
         if (qoff >= inf.rows) { qoff = 0; ++r; }
         if (r < p.ratio) {
@@ -543,7 +562,10 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
       }
       qb = kept_base + __builtin_ctzll(kept);
       kept &= kept - 1;
-      inf = p.info[qb];
+      // the q block's geometry follows from the sequence's (no load on this path)
+      inf.q_pos = (qb - qb_begin) * p.qbs;
+      inf.row_begin = seq_row0 + inf.q_pos;
+      inf.rows = min(p.qbs, seq_qlen - inf.q_pos);
       r = 0;
       qoff = -64;
     }
