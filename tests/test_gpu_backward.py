@@ -63,6 +63,8 @@ CASES = [
     (6, [512, 1000], [512, 1000], 8, 8, 128, 128, 128, 0.3, True, None),
     (7, [200, 1], [1, 333], 8, 1, 64, 80, 48, 0.7, False, -0.1),
     (8, [33, 77, 190], [190, 33, 77], 2, 2, 32, 16, 16, 0.4, True, None),
+    (9, [700, 130], [130, 700], 4, 1, 128, 256, 16, 0.5, True, None),
+    (10, [513], [1029], 2, 2, 128, 64, 192, 0.5, False, None),
 ]
 
 
