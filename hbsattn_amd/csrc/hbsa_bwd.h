@@ -8,7 +8,7 @@
 //     dV = P^T dO      dP = dO V^T      dS = P * (dP - delta)
 //     dQ = scale * dS K                 dK = scale * dS^T Q
 //
-// Three kernels, no atomics, every output element written by exactly one workgroup:
+// Three launches per call, no atomics, every output element written by exactly one workgroup:
 //   hbsa_bwd_delta_kernel : delta[row, q head] = sum_d dO * O
 //   hbsa_bwd_dq_kernel    : one workgroup per (kv head, q block, group of four 32-row wave slots), the
 //                           forward's decomposition; walks the kept k blocks of the q block's bit row.
@@ -21,7 +21,8 @@
 //                           registers, the Q and dO rows of every q block that keeps the k block (and of
 //                           every q head of the group) stream through LDS in 64-row tiles:
 //                           S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS.
-// Both recompute S.  A tile goes from global memory to registers while the tile before it is computed
+// Both recompute S.  The kept blocks of a mask row or column are found with one load per 32 or 64
+// blocks, not one per block.  A tile goes from global memory to registers while the tile before it is computed
 // on, and from registers to LDS between two barriers; a tile that is read both by rows and transposed
 // is stored twice, once in each of the forward's two swizzled layouts.  The forward's persistent
 // scheduling and LDS-DMA double buffering are not applied here yet.
