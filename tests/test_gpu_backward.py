@@ -3,7 +3,8 @@ operator) against the float32 gradient oracle (``oracle.grads``) on the same see
 
 The reference has no backward to compare with (reference ``hbsattn/hbsa_interface.py:31-32``); the
 oracle is pinned in ``tests/test_oracle_grads.py``.  Tolerance for 16-bit tensors against float32:
-max-abs error at most 1e-2 of the largest gradient magnitude (at least 1), mean-abs at most 2e-3.
+max-abs error at most 1e-2 of the largest gradient magnitude (at least 1), mean-abs at most 2e-3 or 1e-2
+of the mean gradient magnitude, whichever is larger.
 """
 import pytest
 import torch
@@ -15,6 +16,7 @@ pytestmark = pytest.mark.gpu
 
 MAX_REL_TOL = 1e-2
 MEAN_ABS_TOL = 2e-3
+MEAN_REL_TOL = 1e-2   # of the mean gradient magnitude, where that is the larger bound (sharp softmax, large gradients)
 
 
 def _problem(seed, q_lens, k_lens, hq, hk, d, qbs, kbs, keep, dtype):
@@ -50,7 +52,8 @@ def _check(got, ref, what):
     err = (got - ref).abs()
     lim = MAX_REL_TOL * max(1.0, ref.abs().max().item())
     assert err.max().item() <= lim, f"{what}: max-abs {err.max().item():.3e} > {lim:.3e}"
-    assert err.mean().item() <= MEAN_ABS_TOL, f"{what}: mean-abs {err.mean().item():.3e} > {MEAN_ABS_TOL}"
+    mean_lim = max(MEAN_ABS_TOL, MEAN_REL_TOL * ref.abs().mean().item())
+    assert err.mean().item() <= mean_lim, f"{what}: mean-abs {err.mean().item():.3e} > {mean_lim:.3e}"
 
 
 CASES = [
@@ -137,3 +140,30 @@ def test_float32_inputs_still_raise_like_the_reference():
     out = HBSAttention(qd, k.cuda(), v.cuda(), cq, ck, mask.cuda(), 32, 32, False, None)
     with pytest.raises(NotImplementedError):
         out.backward(do.cuda())
+
+
+def test_seeded_random_shapes_against_the_gradient_oracle():
+    import random
+    rng = random.Random(4242)
+    for case in range(32):
+        batch = rng.randint(1, 3)
+        q_lens = [rng.randint(1, 500) for _ in range(batch)]
+        k_lens = q_lens if rng.random() < 0.3 else [rng.randint(1, 600) for _ in range(batch)]
+        hk = rng.choice([1, 2, 3])
+        ratio = rng.choice([1, 1, 2, 4])
+        d = rng.choice([16, 32, 40, 64, 96, 128, 128])
+        qbs = 16 * rng.randint(1, 12)
+        kbs = 16 * rng.randint(1, 12)
+        dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+        causal = rng.random() < 0.6
+        scale = rng.choice([None, None, 0.05, 0.3])
+        keep = rng.choice([0.15, 0.5, 0.9, 1.1])
+        what = (f"case {case}: q={q_lens} k={k_lens} heads={hk * ratio}/{hk} d={d} blocks={qbs}x{kbs} {dtype} "
+                f"causal={causal} scale={scale} keep={keep}")
+        print("backward random " + what, flush=True)
+        q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(7000 + case, q_lens, k_lens, hk * ratio, hk, d, qbs, kbs, keep, dtype)
+        _, dq, dk, dv = _gpu_grads(q, k, v, do, cq, ck, mask, qbs, kbs, causal, scale)
+        rdq, rdk, rdv = hbsa_oracle_grads(q, k, v, do, cu_q, cu_k, mask, qbs, kbs, causal, scale)
+        _check(dq, rdq, what + " dq")
+        _check(dk, rdk, what + " dk")
+        _check(dv, rdv, what + " dv")
