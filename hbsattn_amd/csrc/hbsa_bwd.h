@@ -37,7 +37,7 @@ struct BwdParams {
   const uint32_t *bits;
   const int32_t *cu_k, *cu_num_q_block, *cu_num_k_block;
   int64_t q_s, q_h, k_s, k_h, v_s, v_h, do_s, do_h, dq_s, dq_h, dk_s, dk_h, dv_s, dv_h;   // bytes
-  int32_t nqb, batch, ratio, nhead_q, qbs, kbs, wpr, causal;
+  int32_t nqb, nkb, xcd_heads, batch, ratio, nhead_q, qbs, kbs, wpr, causal;   // xcd_heads: see the dK/dV kernels
   int32_t wps, nsub;     // q side: wave slots per q head and workgroups per (kv head, q block), as in the forward
   int32_t nsub_k;        // k side: workgroups per (kv head, k block) = ceil(k_block_size / 128)
   float c;               // softmax_scale * log2(e), signed
@@ -307,8 +307,17 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g32 = lane >> 5, l32 = lane & 31;
-  const int hk = blockIdx.y;
-  const int kb = blockIdx.x / p.nsub_k, sub = blockIdx.x - kb * p.nsub_k;
+  // With a multiple of eight kv heads the grid is one-dimensional and workgroup ids, which go round the
+  // eight XCDs (each with its own L2), are decoded so that XCD x works on the heads x, x + 8, ...: the
+  // workgroups that share an L2 then walk the k blocks of one head in order and read the Q and dO rows of
+  // one sequence at a time, and every XCD has the same amount of work whatever the sequence lengths.
+  int hk = blockIdx.y, bx = blockIdx.x;
+  if (p.xcd_heads) {
+    const unsigned t = blockIdx.x >> 3, per_head = (unsigned)(p.nkb * p.nsub_k);
+    hk = (int)(blockIdx.x & 7u) + 8 * (int)(t / per_head);
+    bx = (int)(t % per_head);
+  }
+  const int kb = bx / p.nsub_k, sub = bx - kb * p.nsub_k;
 
   int b = 0;   // the sequence the k block belongs to
   while (b + 1 < p.batch && p.cu_num_k_block[b + 1] <= kb) ++b;
@@ -493,8 +502,17 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slot = wave & 3, half = wave >> 2;   // 32-key slot of the workgroup; which 32 rows of a tile
   const int g32 = lane >> 5, l32 = lane & 31;
-  const int hk = blockIdx.y;
-  const int kb = blockIdx.x / p.nsub_k, sub = blockIdx.x - kb * p.nsub_k;
+  // With a multiple of eight kv heads the grid is one-dimensional and workgroup ids, which go round the
+  // eight XCDs (each with its own L2), are decoded so that XCD x works on the heads x, x + 8, ...: the
+  // workgroups that share an L2 then walk the k blocks of one head in order and read the Q and dO rows of
+  // one sequence at a time, and every XCD has the same amount of work whatever the sequence lengths.
+  int hk = blockIdx.y, bx = blockIdx.x;
+  if (p.xcd_heads) {
+    const unsigned t = blockIdx.x >> 3, per_head = (unsigned)(p.nkb * p.nsub_k);
+    hk = (int)(blockIdx.x & 7u) + 8 * (int)(t / per_head);
+    bx = (int)(t % per_head);
+  }
+  const int kb = bx / p.nsub_k, sub = bx - kb * p.nsub_k;
 
   int b = 0;   // the sequence the k block belongs to
   while (b + 1 < p.batch && p.cu_num_k_block[b + 1] <= kb) ++b;
@@ -709,11 +727,13 @@ int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_
   }
   hipLaunchKernelGGL((hbsa_bwd_dq_kernel<D, E>), dim3((unsigned)(bp.nqb * bp.nsub), (unsigned)nhead_k), dim3(kThreads), lds_dq,
                      stream, bp);
+  const dim3 kv_grid = bp.xcd_heads ? dim3((unsigned)(num_k_block * bp.nsub_k * nhead_k))
+                                    : dim3((unsigned)(num_k_block * bp.nsub_k), (unsigned)nhead_k);
   if constexpr (D == 128) {
-    hipLaunchKernelGGL((hbsa_bwd_dkv8_kernel<E>), dim3((unsigned)(num_k_block * bp.nsub_k), (unsigned)nhead_k), dim3(512),
+    hipLaunchKernelGGL((hbsa_bwd_dkv8_kernel<E>), kv_grid, dim3(512),
                        lds_dkv, stream, bp);
   } else {
-    hipLaunchKernelGGL((hbsa_bwd_dkv_kernel<D, E>), dim3((unsigned)(num_k_block * bp.nsub_k), (unsigned)nhead_k),
+    hipLaunchKernelGGL((hbsa_bwd_dkv_kernel<D, E>), kv_grid,
                        dim3(kThreads), lds_dkv, stream, bp);
   }
   const hipError_t e = hipGetLastError();

@@ -68,6 +68,8 @@ CASES = [
     (8, [33, 77, 190], [190, 33, 77], 2, 2, 32, 16, 16, 0.4, True, None),
     (9, [700, 130], [130, 700], 4, 1, 128, 256, 16, 0.5, True, None),
     (10, [513], [1029], 2, 2, 128, 64, 192, 0.5, False, None),
+    (11, [200, 150], [180, 260], 16, 8, 64, 64, 64, 0.5, True, None),     # eight kv heads: the grid decoded by XCD
+    (12, [300], [300], 16, 16, 128, 128, 128, 0.6, True, None),
 ]
 
 
