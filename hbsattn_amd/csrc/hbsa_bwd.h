@@ -191,9 +191,15 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int g32 = lane >> 5, l32 = lane & 31;
-  const int hk = blockIdx.y;
+  // (grid decoding by XCD: see hbsa_bwd_dkv_kernel)
+  int hk = blockIdx.y, bx = blockIdx.x;
+  if (p.xcd_heads) {
+    const unsigned t = blockIdx.x >> 3, per_head = (unsigned)(p.nqb * p.nsub);
+    hk = (int)(blockIdx.x & 7u) + 8 * (int)(t / per_head);
+    bx = (int)(t % per_head);
+  }
   // last q blocks first: under a causal mask they are the long ones, and the grid should not end on them
-  const int qb_rev = blockIdx.x / p.nsub, sub = blockIdx.x - qb_rev * p.nsub;
+  const int qb_rev = bx / p.nsub, sub = bx - qb_rev * p.nsub;
   const int qb = p.nqb - 1 - qb_rev;
   const QBlockInfo inf = p.info[qb];
 
@@ -725,8 +731,8 @@ int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_
       raised[dev] = true;
     }
   }
-  hipLaunchKernelGGL((hbsa_bwd_dq_kernel<D, E>), dim3((unsigned)(bp.nqb * bp.nsub), (unsigned)nhead_k), dim3(kThreads), lds_dq,
-                     stream, bp);
+  const dim3 q_grid = bp.xcd_heads ? dim3((unsigned)(bp.nqb * bp.nsub * nhead_k)) : dim3((unsigned)(bp.nqb * bp.nsub), (unsigned)nhead_k);
+  hipLaunchKernelGGL((hbsa_bwd_dq_kernel<D, E>), q_grid, dim3(kThreads), lds_dq, stream, bp);
   const dim3 kv_grid = bp.xcd_heads ? dim3((unsigned)(num_k_block * bp.nsub_k * nhead_k))
                                     : dim3((unsigned)(num_k_block * bp.nsub_k), (unsigned)nhead_k);
   if constexpr (D == 128) {

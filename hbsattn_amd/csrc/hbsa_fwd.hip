@@ -1798,12 +1798,14 @@ int hbsa_bwd(const void *q, const void *k, const void *v, const void *out, const
   bp.dq_s = strides[10] * es; bp.dq_h = strides[11] * es; bp.dk_s = strides[12] * es; bp.dk_h = strides[13] * es;
   bp.dv_s = strides[14] * es; bp.dv_h = strides[15] * es;
   bp.nqb = num_q_block; bp.nkb = num_k_block; bp.batch = batch;
-  bp.xcd_heads = (nhead_k % 8 == 0 && (long long)num_k_block * ((k_block_size + 127) / 128) * nhead_k < (1LL << 31)) ? 1 : 0; bp.ratio = nhead_q / nhead_k; bp.nhead_q = nhead_q; bp.qbs = q_block_size;
+  bp.ratio = nhead_q / nhead_k; bp.nhead_q = nhead_q; bp.qbs = q_block_size;
   bp.kbs = k_block_size;
   bp.wpr = words_per_row(num_k_block); bp.causal = causal ? 1 : 0;
   bp.wps = (q_block_size + kWaveRows - 1) / kWaveRows;
   bp.nsub = (bp.ratio * bp.wps + 3) / 4;
   bp.nsub_k = (k_block_size + 4 * kWaveRows - 1) / (4 * kWaveRows);
+  bp.xcd_heads = (nhead_k % 8 == 0 && (long long)num_k_block * bp.nsub_k * nhead_k < (1LL << 31) &&
+                  (long long)num_q_block * bp.nsub * nhead_k < (1LL << 31)) ? 1 : 0;
   bp.c = softmax_scale * kLog2e;
   bp.scale = softmax_scale;
   DeltaParams dp;
