@@ -6,12 +6,13 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhbsattn_amd.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 DTYPE_BF16 = 0
 DTYPE_F16 = 1
 DTYPE_F32 = 2
 DTYPE_F32_STAGED16 = 3
+STATIC_SCRATCH_BYTES = 32 << 20   # HBSA_STATIC_SCRATCH_BYTES of include/hbsattn_amd.h
 
 _lib = None
 
@@ -45,6 +46,8 @@ def load() -> ctypes.CDLL:
     lib.hbsa_fwd.argtypes = ([vp] * 11 + [ctypes.c_size_t] + [ctypes.c_int32] * 12 + [ctypes.c_float]
                              + [ctypes.POINTER(ctypes.c_int64), vp])
     i64p = ctypes.POINTER(ctypes.c_int64)
+    lib.hbsa_fwd_static.restype = ctypes.c_int
+    lib.hbsa_fwd_static.argtypes = [vp] * 10 + [ctypes.c_int32] * 12 + [ctypes.c_float, i64p, vp]
     lib.hbsa_fwd_prepare.restype = ctypes.c_int
     lib.hbsa_fwd_prepare.argtypes = [vp] * 7 + [ctypes.c_size_t] + [ctypes.c_int32] * 7 + [i64p, vp]
     lib.hbsa_fwd_run.restype = ctypes.c_int

@@ -31,6 +31,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <type_traits>
 
 #include "hbsattn_amd.h"
@@ -1746,6 +1747,54 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32
                       num_q_block, num_k_block, q_block_size, k_block_size, causal, softmax_scale, strides, stream);
 }
 
+// ---- hbsa_fwd without a workspace argument: the work description lives in this array.  Every GPU
+// the library runs on holds its own copy at its own address until the process ends.  In host code
+// the array's name is only a handle; its device address comes from hipGetSymbolAddress, once per
+// device, and is what the kernels receive.
+}  // extern "C"
+static __device__ __align__(256) unsigned char scratch[HBSA_STATIC_SCRATCH_BYTES];
+namespace {
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void **ptr) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail((int)e, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(HBSA_ERR_UNSUPPORTED, "device index above %d", kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) return fail(e != hipSuccess ? (int)e : HBSA_ERR_UNSUPPORTED, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+}  // namespace
+extern "C" {
+
+int hbsa_fwd_static(const void *q, const void *k, const void *v, void *out, const int32_t *cu_q_seqlens,
+                    const int32_t *cu_k_seqlens, const uint8_t *block_mask, const int32_t *q_block_to_batch,
+                    const int32_t *cu_num_q_block, const int32_t *cu_num_k_block, int32_t dtype, int32_t batch,
+                    int32_t total_q, int32_t total_k, int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+                    int32_t num_q_block, int32_t num_k_block, int32_t q_block_size, int32_t k_block_size, int32_t causal,
+                    float softmax_scale, const int64_t *strides, void *stream) {
+  g_err[0] = 0;
+  if (total_q == 0 || num_q_block == 0 || nhead_q == 0) return 0;
+  const size_t need = hbsa_fwd_workspace_bytes_dtype(dtype, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
+                                                     num_k_block);
+  if (need > (size_t)HBSA_STATIC_SCRATCH_BYTES)
+    return fail(HBSA_ERR_WORKSPACE_TOO_SMALL,
+                "this problem needs %zu bytes of scratch, hbsa_fwd_static holds %zu: use hbsa_fwd with a workspace", need,
+                (size_t)HBSA_STATIC_SCRATCH_BYTES);
+  void *ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  return hbsa_fwd(q, k, v, out, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_to_batch, cu_num_q_block, cu_num_k_block, ws,
+                  (size_t)HBSA_STATIC_SCRATCH_BYTES, dtype, batch, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
+                  num_k_block, q_block_size, k_block_size, causal, softmax_scale, strides, stream);
+}
 
 size_t hbsa_bwd_workspace_bytes(int32_t total_q, int32_t nhead_q) {
   if (total_q < 0 || nhead_q < 0) return 0;

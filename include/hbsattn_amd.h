@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define HBSA_ABI_VERSION 3
+#define HBSA_ABI_VERSION 4
 
 /* element types of q/k/v/out (reference: dtype follows the input tensors,
  * hbsattn/fwd_triton_auto_tile_size.py:272) */
@@ -139,6 +139,32 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out,
              int32_t q_block_size, int32_t k_block_size,
              int32_t causal, float softmax_scale,
              const int64_t *strides, void *stream);
+
+/*
+ * hbsa_fwd for callers that cannot allocate device memory or pass a workspace: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (whose launcher allocates its scratch with torch on every call, reference
+ * hbsattn/fwd_triton_auto_tile_size.py:273-274).  Same arguments and results as hbsa_fwd without
+ * `workspace` / `workspace_bytes`: the work description lives in a device array of
+ * HBSA_STATIC_SCRATCH_BYTES inside the library, which every GPU the library runs on holds until the
+ * process ends.  The call allocates and frees nothing.  A problem whose
+ * hbsa_fwd_workspace_bytes_dtype(...) exceeds HBSA_STATIC_SCRATCH_BYTES is refused with
+ * HBSA_ERR_WORKSPACE_TOO_SMALL before anything is launched.  All calls on one GPU share that GPU's
+ * array: calls on one stream are ordered and safe; calls that overlap on one GPU (different streams
+ * or host threads) race on it and must be serialised by the caller.
+ */
+#define HBSA_STATIC_SCRATCH_BYTES (32u << 20)
+int hbsa_fwd_static(const void *q, const void *k, const void *v, void *out,
+                    const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens,
+                    const uint8_t *block_mask,
+                    const int32_t *q_block_to_batch, const int32_t *cu_num_q_block,
+                    const int32_t *cu_num_k_block,
+                    int32_t dtype, int32_t batch, int32_t total_q, int32_t total_k,
+                    int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+                    int32_t num_q_block, int32_t num_k_block,
+                    int32_t q_block_size, int32_t k_block_size,
+                    int32_t causal, float softmax_scale,
+                    const int64_t *strides, void *stream);
 
 /*
  * The two halves of hbsa_fwd, for callers that apply one block mask to many q/k/v
