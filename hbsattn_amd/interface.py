@@ -67,7 +67,10 @@ def _pad_headdim(t: torch.Tensor, d_pad: int) -> torch.Tensor:
 class PreparedMask:
     """Result of the pre-pass for one (block_mask, sequence boundaries, block sizes, causal)
     combination: the device scratch the attention kernel reads.  Reusable across calls that
-    share those, e.g. the layers of a model that share one sparsity pattern."""
+    share those, e.g. the layers of a model that share one sparsity pattern, as long as those calls
+    are ordered on ONE stream: the scratch also holds per-launch state (work-queue counters, softmax
+    constants, staging copies and split partials), so two ``hbsa_run`` calls on one ``PreparedMask``
+    that overlap on different streams corrupt each other."""
 
     def __init__(self, workspace, nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, causal,
                  cu_k_seqlens=None, cu_num_q_block=None, cu_num_k_block=None):
@@ -82,6 +85,15 @@ class PreparedMask:
         self.q_block_size = q_block_size
         self.k_block_size = k_block_size
         self.causal = bool(causal)
+
+
+def _check_on_device(dev, **tensors):
+    """The kernels dereference these pointers on ``dev``: a host tensor, or one on another GPU, would be
+    a memory fault there, not an exception."""
+    for name, t in tensors.items():
+        if not isinstance(t, torch.Tensor) or t.device != dev:
+            where = t.device if isinstance(t, torch.Tensor) else type(t).__name__
+            raise RuntimeError(f"{name} must be a tensor on {dev} (the device of block_mask), not on {where}")
 
 
 def _check_block_sizes(q_block_size, k_block_size):
@@ -119,8 +131,19 @@ def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_s
     if not block_mask.is_cuda:
         raise RuntimeError("hbsattn_amd runs on MI355X only: block_mask must be a CUDA(HIP) tensor; there is no CPU path")
     _check_block_sizes(q_block_size, k_block_size)
-    lib = _lib.load()
+    if block_mask.dtype != torch.bool:
+        raise TypeError(f"block_mask must be a boolean tensor, not {block_mask.dtype}")
+    if block_mask.dim() != 3 or tuple(block_mask.shape[1:]) != (int(num_q_block), int(num_k_block)):
+        raise ValueError("block_mask must have shape (nheads_k, num_q_block, num_k_block) = "
+                         f"(*, {int(num_q_block)}, {int(num_k_block)}), not {tuple(block_mask.shape)}")
     dev = block_mask.device
+    _check_on_device(dev, cu_q_seqlens=cu_q_seqlens, cu_k_seqlens=cu_k_seqlens, q_block_to_batch=q_block_to_batch,
+                     cu_num_q_block=cu_num_q_block, cu_num_k_block=cu_num_k_block)
+    if cu_q_seqlens.numel() != cu_k_seqlens.numel() or cu_num_q_block.numel() != cu_q_seqlens.numel() \
+            or cu_num_k_block.numel() != cu_q_seqlens.numel() or q_block_to_batch.numel() != int(num_q_block):
+        raise ValueError("sequence boundaries and block metadata disagree in length (batch + 1 entries each, "
+                         "num_q_block entries in q_block_to_batch)")
+    lib = _lib.load()
     nhead_k = block_mask.shape[0]
     ws_bytes = int(lib.hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block))
     if run_shape is not None:
@@ -146,7 +169,8 @@ def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_s
 
 def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = False):
     """Runs the attention kernel (``hbsa_fwd_run`` / ``hbsa_fwd_run_lse``) on the current stream from a
-    prepared mask.  With ``return_lse`` the result is ``(out, lse)``, ``lse`` a float32
+    prepared mask (calls that share a ``PreparedMask`` must be ordered on one stream; a call may
+    replace ``prepared.workspace`` by a larger one).  With ``return_lse`` the result is ``(out, lse)``, ``lse`` a float32
     ``[total_q, nhead_q]`` tensor: log of the sum over a row's visible keys of exp(scale * q.k)."""
     if not q.is_cuda:
         raise RuntimeError("hbsattn_amd runs on MI355X only: q/k/v must be CUDA(HIP) tensors; there is no CPU path")
@@ -222,6 +246,7 @@ def hbsa_backward(q, k, v, out, dout, lse, prepared: PreparedMask, softmax_scale
         raise NotImplementedError("hbsattn_amd: the backward takes bfloat16 / float16 tensors with headdim <= 128")
     if prepared.cu_k_seqlens is None:
         raise ValueError("this PreparedMask was built without the sequence boundaries the backward needs")
+    _check_on_device(prepared.workspace.device, q=q, k=k, v=v, out=out, dout=dout, lse=lse)
     lib = _lib.load()
     total_q, nhead_q, headdim = q.shape
     total_k, nhead_k = k.shape[0], k.shape[1]

@@ -1,4 +1,9 @@
-"""The committed fixtures of tests/golden (written by tests/golden/make_fixtures.py)."""
+"""The committed fixtures of tests/golden (written by tests/golden/make_fixtures.py).
+
+``readme_calculate_blocks.json`` is the worked example the reference's README prints (a vector the
+reference itself holds).  ``small_problems.npz`` is NOT a reference-held vector: its outputs were written
+by this repository's own C oracle (``oracle/scalar.c``), so it is a drift guard for the oracle and the
+kernels, and pins nothing independently; what pins the oracle is in tests/test_oracle_*.py."""
 import json
 import os
 

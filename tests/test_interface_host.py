@@ -90,3 +90,33 @@ def test_fp32_mode_switch_validates_and_returns_the_previous_mode():
         assert interface._fp32_mode == "exact"
     finally:
         set_fp32_mode(first)
+
+
+def test_prepare_rejects_host_metadata_and_bad_masks_before_any_launch():
+    """Sequence boundaries or block metadata on the host (or a mask of the wrong dtype / shape) must raise:
+    their pointers would be dereferenced on the GPU.  A fake device mask stands in for a GPU tensor; the
+    checks run before the library is loaded or anything is launched."""
+    from hbsattn_amd import interface
+
+    class FakeMask:
+        is_cuda = True
+        dtype = torch.bool
+        shape = (2, 5, 12)
+        device = torch.device("cuda", 0)
+
+        def dim(self):
+            return 3
+
+    q, k, v, cu_q, cu_k, mask = _toy()
+    nq, _, qb2b, cu_nqb = hbsattn_amd.calculate_blocks(cu_q, 32)
+    nk, _, _, cu_nkb = hbsattn_amd.calculate_blocks(cu_k, 16)
+    with pytest.raises(RuntimeError, match="cu_q_seqlens must be a tensor on cuda:0"):
+        interface.hbsa_prepare(cu_q, cu_k, FakeMask(), 32, 16, True, nq, qb2b, cu_nqb, nk, cu_nkb)
+    bad = FakeMask()
+    bad.dtype = torch.uint8
+    with pytest.raises(TypeError, match="boolean"):
+        interface.hbsa_prepare(cu_q, cu_k, bad, 32, 16, True, nq, qb2b, cu_nqb, nk, cu_nkb)
+    bad = FakeMask()
+    bad.shape = (2, 5, 11)
+    with pytest.raises(ValueError, match=r"\(\*, 5, 12\)"):
+        interface.hbsa_prepare(cu_q, cu_k, bad, 32, 16, True, nq, qb2b, cu_nqb, nk, cu_nkb)
