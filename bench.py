@@ -1,7 +1,10 @@
 #!/usr/bin/env python3
 """Benchmark of the block-sparse attention forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|T|C3|C4|C5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload T|C2|C3|C4|C5]
+
+The default workload is T, the shape the 50 %-of-peak goal is stated on; C2 and C4 are measured
+after it and reported under ``other_shapes``.
 
 A step is one ``HBSAttention`` call (pre-pass + attention kernel, block metadata
 pre-computed and passed in as the reference's sweep does, reference
@@ -33,6 +36,7 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, vendor figure
+RIDGE_FLOP_PER_BYTE = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
 
 DESCRIPTIONS = {
     "C2": "C2: batch 8 x 8192 tokens, Hq=Hk=32, D=128, 128x128 blocks, keep 0.1 + diagonal, causal, bf16",
@@ -41,14 +45,41 @@ DESCRIPTIONS = {
     "C4": "C4: batch 8 x 65536 tokens, Hq=Hk=32, D=128, 128x128 blocks, keep 0.3, non-causal, bf16",
     "C5": "C5: q lens 3000/5120/777/4096, k lens 6000/5120/4100/8192, Hq=16 Hk=2, D=64, 80x48 blocks, keep 0.5, causal, scale 0.1, bf16",
 }
-# which roof bounds the attention kernel at each workload (arithmetic intensity against the
-# ridge at 2500 TFLOP/s / 8 TB/s = 312 FLOP/B)
-BOUND = {"C2": "hbm", "T": "mfma", "C3": "mfma", "C4": "mfma", "C5": "hbm"}
-# HBM bytes per launch of the attention kernel, from rocprofv3 counter runs of this program
-# (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, scaled by what the same counters read for a
-# 1 GiB device-to-device copy: factors 2.000 and 1.000).  Not measured live: a counter run needs
-# the profiler.  The summaries are under profiles/.
-MEASURED_TRAFFIC_BYTES = {"C2": 4.87e9, "T": 56.6e9}
+SHAPES = {"C2": "B8 H32 D128 L=8K", "T": "B8 H32 D128 L=32K", "C3": "B8 Hq32/Hk8 D128 varlen", "C4": "B8 H32 D128 L=64K",
+          "C5": "B4 Hq16/Hk2 D64 q!=k"}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def kernel_sources_sha16() -> str:
+    """Content hash of the kernel sources (hbsattn_amd/csrc): what a counter measurement belongs to."""
+    import hashlib
+
+    h = hashlib.sha256()
+    d = os.path.join(ROOT, "hbsattn_amd", "csrc")
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".h", ".cpp")):
+            h.update(name.encode())
+            with open(os.path.join(d, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(name):
+    """HBM bytes per launch of the attention kernel for a workload, from profiles/traffic.json: rocprofv3
+    counter runs of this program (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, scaled by what the same
+    counters read for a 1 GiB device-to-device copy).  A counter run needs the profiler, so the figure is
+    read, not measured live; it is dropped when the kernel sources have changed since it was taken."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None, "profiles/traffic.json missing"
+    entry = table.get("workloads", {}).get(name)
+    if entry is None:
+        return None, "no counter run for this workload"
+    if table.get("kernel_sources_sha16") != kernel_sources_sha16():
+        return None, f"stale: counters were taken at kernel sources {table.get('kernel_sources_sha16')}"
+    return float(entry["bytes"]), entry.get("profile", "")
 
 
 def time_steps(fn, steps, warmup):
@@ -113,16 +144,20 @@ def measure(name, steps, warmup):
         "bytes": work["bytes"],
         "visited_pairs": work["visited_pairs"],
     }
-    if BOUND[name] == "mfma":
+    traffic, traffic_note = measured_traffic(name)
+    intensity = work["flops"] / work["bytes"]
+    if intensity >= RIDGE_FLOP_PER_BYTE:   # right of the ridge at 2500 TFLOP/s / 8 TB/s = 312.5 FLOP/B
         ach = work["flops"] / kernel_ms / 1e9
         res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                           "frac": ach / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": "hbsa_fwd_kernel",
-                           "kernel_ms": kernel_ms, "algorithmic_flops": work["flops"]}
+                           "frac": ach / PEAK_BF16_TFLOPS, "traffic": traffic, "traffic_from_profile": traffic_note,
+                           "kernel": "hbsa_fwd_kernel", "kernel_ms": kernel_ms, "algorithmic_flops": work["flops"],
+                           "flop_per_byte": intensity}
     else:
         ach = work["bytes"] / kernel_ms / 1e6
         res["roofline"] = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                           "frac": ach / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": "hbsa_fwd_kernel",
-                           "kernel_ms": kernel_ms, "algorithmic_bytes": work["bytes"],
+                           "frac": ach / PEAK_HBM_GBS, "traffic": traffic, "traffic_from_profile": traffic_note,
+                           "kernel": "hbsa_fwd_kernel", "kernel_ms": kernel_ms, "algorithmic_bytes": work["bytes"],
+                           "flop_per_byte": intensity,
                            "mfma_frac": work["flops"] / kernel_ms / 1e9 / PEAK_BF16_TFLOPS}
     return w, res
 
@@ -193,9 +228,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=sorted(DESCRIPTIONS))
+    ap.add_argument("--workload", default="T", choices=sorted(DESCRIPTIONS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-target", action="store_true", help="skip the extra measurement at the 32K target shape")
+    ap.add_argument("--no-others", action="store_true",
+                    help="skip the extra measurements at the other full-size shapes (reported under 'other_shapes')")
+    ap.add_argument("--others", default="C2,C4", help="comma-separated workloads measured besides --workload")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--backward", action="store_true", help="also time the backward kernels (reported under 'backward')")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -219,7 +256,7 @@ def main():
 
     w, res = measure(a.workload, a.steps, a.warmup)
     line = {
-        "metric": "effective TFLOP/s over kept blocks, block-sparse attention forward (B8 H32 D128)",
+        "metric": f"effective TFLOP/s over kept blocks, block-sparse attention forward ({SHAPES[a.workload]})",
         "value": res["tflops"],
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -232,22 +269,29 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": DESCRIPTIONS[a.workload], "timing": "K calls between two synchronisations, "
-                   "block metadata precomputed; pre-pass + attention kernel per call"},
+                   "block metadata precomputed; one HBSAttention call per step"},
         "roofline": res["roofline"],
         "detail": {k: res[k] for k in ("per_call_sync_ms", "attention_kernel_ms", "prepass_ms", "tflops_exact_elements",
                                        "flops", "bytes", "visited_pairs")},
     }
+    if a.workload == "T":
+        line["goal"] = ">= 0.50 of bf16 dense MFMA peak at this shape"
     if a.backward:
         line["backward"] = measure_backward(w, res["flops"], max(1, a.steps // 5))
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w, a.cpu_budget)
     del w
     torch.cuda.empty_cache()
-    if not a.no_target and a.workload != "T":
-        _, t = measure("T", a.steps, a.warmup)
-        line["target_shape"] = {"workload": DESCRIPTIONS["T"], "ms_per_step": t["ms_per_step"], "tflops": t["tflops"],
-                                "attention_kernel_ms": t["attention_kernel_ms"], "roofline": t["roofline"],
-                                "goal": ">= 0.50 of bf16 dense MFMA peak"}
+    if not a.no_others:
+        line["other_shapes"] = {}
+        for name in [n for n in a.others.split(",") if n and n != a.workload]:
+            heavy = name == "C4"   # 0.2 s per call: a few steps are enough
+            wo, t = measure(name, max(3, a.steps // 5) if heavy else a.steps, min(a.warmup, 2) if heavy else a.warmup)
+            del wo
+            torch.cuda.empty_cache()
+            line["other_shapes"][name] = {"workload": DESCRIPTIONS[name], "ms_per_step": t["ms_per_step"],
+                                          "tflops": t["tflops"], "attention_kernel_ms": t["attention_kernel_ms"],
+                                          "roofline": t["roofline"]}
     print(json.dumps(line))
 
 

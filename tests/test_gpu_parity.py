@@ -509,6 +509,26 @@ def test_few_long_items_are_split_over_key_blocks_and_merged(dtype, d, causal, k
     assert (unsplit.float() - out.float()).abs().max().item() <= 2e-2
 
 
+def test_split_with_fp32_inputs_in_the_fast_mode():
+    """fp32 q/k/v staged as fp16 AND split over key blocks: the merge kernel then applies the staging
+    multiplier of v to its fp32 output."""
+    from hbsattn_amd import _lib, set_fp32_mode
+    previous = set_fp32_mode("fast")
+    try:
+        w = make_problem(seed=83, q_lens=[128, 70], k_lens=[9000, 4000], hq=4, hk=2, d=64, qbs=64, kbs=128, keep=0.6,
+                         diag=True, causal=True, scale=None, dtype=torch.float32)
+        w.v = w.v * 37.5          # a staging multiplier for v other than the one for unit-scale data
+        lib = _lib.load()
+        assert lib.hbsa_fwd_split_workspace_bytes(w.q.shape[0], 4, 2, 64, w.q_meta[0], w.k_meta[0], 64) > 0
+        out, lse = _run_lse(w)
+        ref_out, ref_lse = hbsa_oracle(w.q.cpu(), w.k.cpu(), w.v.cpu(), w.cu_q, w.cu_k, w.block_mask.cpu(), w.q_block_size,
+                                       w.k_block_size, w.causal, w.softmax_scale, return_lse=True)
+        assert_close_to_oracle(out / 37.5, ref_out / 37.5, "split, fp32 fast mode")
+        assert (lse.cpu() - ref_lse).abs().max().item() <= 2e-3
+    finally:
+        set_fp32_mode(previous)
+
+
 def test_split_with_many_kv_heads_and_a_head_count_that_is_no_multiple_of_eight():
     w = make_problem(seed=82, q_lens=[64, 33], k_lens=[5000, 2500], hq=24, hk=12, d=64, qbs=64, kbs=128, keep=0.5, diag=True,
                      causal=True, scale=0.1)
