@@ -79,6 +79,7 @@ struct PrepParams {
   int64_t ms_h, ms_q, ms_k;
   QBlockInfo *info;
   uint32_t *bits;
+  struct Sched *sched;
   int32_t nqb, qbs, kbs, wpr, causal;
 };
 
@@ -108,9 +109,11 @@ struct FwdParams {
   int32_t wps;    // wave slots per q head = ceil(q_block_size / 32)
   int32_t nsub;   // workgroups per (kv head, q block) = ceil(ratio * wps / 4)
   uint32_t q_sign;  // 0x80008000 when softmax_scale < 0 (Q is negated, |scale| used)
-  float c;        // |softmax_scale| * log2(e); the kernel reads the launch's value from sched
+  float c;        // |softmax_scale| * log2(e)
+  float lag;      // kLazyRescaleLog2 / c: how far the running max may lag, in raw score units
   FastDiv div_nsub, div_nqb, div_kbs;   // divisions on the scheduler's path
-  int32_t f32;    // fp32 inputs staged as fp16: the setup kernel derives the constants from the maxima
+  int32_t f32;    // fp32 inputs staged as fp16: the softmax constants come from the launch record, where
+                  // the setup kernel derived them from the tensors' maxima
   int32_t nhead_k;
   struct Sched *sched;
   float *lse;             // optional [total_q, nhead_q] log-sum-exp output (nullptr: none)
@@ -131,6 +134,8 @@ struct FwdParams {
 __global__ __launch_bounds__(kThreads) void hbsa_prep_kernel(PrepParams p) {
   const int lane = threadIdx.x & 63;
   const int g = blockIdx.x * 4 + (threadIdx.x >> 6);
+  // the work-queue counters of the launch record start at zero; every attention launch leaves them so
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < 9) ((uint32_t *)p.sched)[threadIdx.x] = 0;
   if (g >= p.nqb) return;
   const int hk = blockIdx.y;
   const int b = p.q_block_to_batch[g];
@@ -242,22 +247,22 @@ __device__ __forceinline__ float half_sum(float x) {
 // --------------------------------------------------------------------------------------
 struct Sched {
   uint32_t qnext[8];   // next unclaimed entry of each queue
-  // softmax constants the attention kernel reads at its start (written by hbsa_setup_kernel)
-  float c;             // |softmax_scale| * log2(e), divided by the q and k staging multipliers for fp32 inputs
+  uint32_t done;       // workgroups of the running attention launch that have made their last claim
+  // fp32 inputs staged as fp16 only (written by hbsa_setup_kernel, read by the attention kernel at its start):
+  float c;             // |softmax_scale| * log2(e), divided by the q and k staging multipliers
   float lag;           // kLazyRescaleLog2 / c, in raw score units
-  float out_mul;       // fp32 inputs: 1 / (v staging multiplier); 1 otherwise
-  // fp32 inputs only: bit patterns of max|x| over q, k, v and the power-of-two staging multipliers
+  float out_mul;       // 1 / (v staging multiplier)
+  // bit patterns of max|x| over q, k, v and the power-of-two staging multipliers
   uint32_t amax[3];
   float in_mul[3];
-  uint32_t pad[47];
+  uint32_t pad[46];
 };
 static_assert(sizeof(Sched) == 256, "Sched is one 256-byte slot of the workspace");
 
-// Queue counters and softmax constants for one attention launch (a kernel, not a memset, so that
-// the launches of a call can be captured in a graph).  For fp32 inputs the constants follow from
-// the maxima the absmax kernels left in s->amax.
+// Softmax constants of an attention launch on fp32 inputs staged as fp16: they follow from the maxima
+// the absmax kernels left in s->amax.  (Launches on 16-bit inputs carry their constants as kernel
+// arguments and need no such step.)
 __global__ void hbsa_setup_kernel(Sched *s, float c, int f32) {
-  if (threadIdx.x < 8) s->qnext[threadIdx.x] = 0;
   if (threadIdx.x != 0) return;
   float out_mul = 1.f;
   if (f32) {
@@ -486,11 +491,29 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   const int g32 = lane >> 5;   // which half of the wavefront
   const int l32 = lane & 31;   // query within the wave slot / key row within a sub-tile
 
-  // softmax constants of this launch (uniform; written by the setup kernel that precedes it)
-  const float sm_c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, p.sched->c)));
-  const float sm_lag = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, p.sched->lag)));
-  const float sm_out_mul =
-      __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, p.sched->out_mul)));
+  // softmax constants of this launch (uniform): kernel arguments, or for fp32 inputs staged as fp16 what
+  // the setup kernel that precedes this launch derived on the device
+  float sm_c = p.c, sm_lag = p.lag, sm_out_mul = 1.f;
+  if (p.f32) {
+    sm_c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, p.sched->c)));
+    sm_lag = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, p.sched->lag)));
+    sm_out_mul = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, p.sched->out_mul)));
+  }
+  // Leaving: wavefront 0 makes every claim of its workgroup.  Once its last claim has been performed it
+  // counts the workgroup as done, and the workgroup that completes the count puts the queue counters
+  // back to zero, so the next launch on this work description needs no preparation of its own.
+  auto leave = [&]() {
+    if (wave != 0) return;
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this workgroup's last claim has returned
+    if (lane == 0) {
+      const uint32_t before = atomicAdd(&p.sched->done, 1u);
+      if (before + 1 == gridDim.x) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) atomicExch(&p.sched->qnext[i], 0u);
+        atomicExch(&p.sched->done, 0u);
+      }
+    }
+  };
 
   // ------------------------------------------------------------------ scheduler (wavefront 0)
   const int nq = p.nhead_k < 8 ? p.nhead_k : 8;                       // queues that hold work
@@ -716,7 +739,10 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 
   // ------------------------------------------------------------------ first item
   int c = 0;   // list / header of the current item
-  if (hdr_word(0, H_HK) < 0) return;
+  if (hdr_word(0, H_HK) < 0) {
+    leave();
+    return;
+  }
   {
     const int total0 = hdr_word(0, H_TOTAL);
     if (total0 > 0) {
@@ -1108,6 +1134,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     if (nxt_hk < 0) break;
     c ^= 1;
   }
+  leave();
 }
 
 // Split over key blocks: bit row copy `part` keeps the k blocks [part * n / nparts, (part + 1) * n / nparts)
@@ -1266,7 +1293,6 @@ int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
     if (resident <= 0) return fail(HBSA_ERR_UNSUPPORTED, "could not size the persistent grid");
   }
   const int grid = (int)(items < resident ? items : resident);
-  hipLaunchKernelGGL(hbsa_setup_kernel, dim3(1), dim3(64), 0, stream, fp.sched, fp.c, fp.f32);
   hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32>), dim3(grid), dim3(kThreads), lds_bytes, stream, fp);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail((int)e, "hbsa_fwd_kernel launch: %s", hipGetErrorString(e));
@@ -1569,6 +1595,7 @@ int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens, c
   pp.mask = block_mask; pp.ms_h = mask_strides[0]; pp.ms_q = mask_strides[1]; pp.ms_k = mask_strides[2];
   pp.info = (QBlockInfo *)workspace;
   pp.bits = (uint32_t *)((char *)workspace + bits_offset(num_q_block));
+  pp.sched = (Sched *)((char *)workspace + sched_offset(num_q_block));
   pp.nqb = num_q_block; pp.qbs = q_block_size; pp.kbs = k_block_size; pp.wpr = words_per_row(num_k_block);
   pp.causal = causal ? 1 : 0;
   hipLaunchKernelGGL(hbsa_prep_kernel, dim3((num_q_block + 3) / 4, nhead_k), dim3(kThreads), 0, (hipStream_t)stream, pp);
@@ -1662,6 +1689,7 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
   float c = std::fabs(softmax_scale) * kLog2e;
   if (c < 1e-30f) c = 1e-30f;  // scale 0: uniform weights over the visible keys, and -inf * c stays -inf
   fp.c = c;
+  fp.lag = kLazyRescaleLog2 / c;
   const long long items = (long long)nhead_k * num_q_block * fp.nsub;
   if (items > 0x7fffffffLL) return fail(HBSA_ERR_UNSUPPORTED, "too many work items (%lld)", items);
   // split over key blocks when the items cannot fill the device and the caller's workspace has the room

@@ -178,8 +178,10 @@ int hbsa_fwd_static(const void *q, const void *k, const void *v, void *out,
  *
  * hbsa_fwd_run runs the attention kernel from a prepared `workspace` (same sizes, block
  * sizes and `causal` as the prepare call; q/k/v/out and softmax_scale may differ per call).
- * It rewrites the scheduler counters inside `workspace`, so two runs that share one
- * workspace must be ordered on one stream, not concurrent.
+ * It advances the work-queue counters inside `workspace` (hbsa_fwd_prepare leaves them at zero and
+ * every attention launch puts them back to zero as its last workgroup ends, so a prepared workspace
+ * can be run any number of times with no step in between); two runs that share one workspace must
+ * therefore be ordered on one stream, not concurrent.
  * It replaces the reference `_fwd_kernel` launch (reference
  * hbsattn/fwd_triton_auto_tile_size.py:283-308).
  *   strides       int64[8] = { q_tok, q_head, k_tok, k_head, v_tok, v_head, out_tok, out_head }

@@ -447,6 +447,58 @@ def test_call_can_be_captured_in_a_graph_and_replayed():
             assert torch.equal(captured, eager0)
 
 
+def test_attention_launches_leave_the_work_queues_ready_for_the_next_launch():
+    """One prepared mask, many attention launches: each launch's last workgroup puts the queue counters
+    back, so every run sees the whole work list (bitwise equal results), also when launches of
+    different grids (another head count on the query side) and with the log-sum-exp output alternate."""
+    from hbsattn_amd.interface import hbsa_prepare, hbsa_run
+    w = make_problem(seed=91, q_lens=[1100, 300, 2048], k_lens=[1500, 300, 2048], hq=8, hk=4, d=64, qbs=64, kbs=64,
+                     keep=0.3, diag=True, causal=True, scale=None)
+    prepared = hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, 64, 64, True, w.q_meta[0], w.q_meta[2],
+                            w.q_meta[3], w.k_meta[0], w.k_meta[3])
+    first = hbsa_run(w.q, w.k, w.v, prepared, None)
+    assert_close_to_oracle(first, oracle_for(w), "first launch")
+    q4 = w.q[:, :4].contiguous()
+    first4 = None
+    for i in range(6):
+        out = hbsa_run(w.q, w.k, w.v, prepared, None, return_lse=bool(i & 1))
+        out = out[0] if isinstance(out, tuple) else out
+        assert torch.equal(out, first), f"launch {i}"
+        out4 = hbsa_run(q4, w.k, w.v, prepared, None)        # nhead_q == nhead_k: half the wave slots, another grid
+        first4 = out4 if first4 is None else first4
+        assert torch.equal(out4, first4), f"launch {i}, 4 q heads"
+
+
+def test_prepared_masks_are_reused_only_for_unchanged_tensors():
+    from hbsattn_amd import interface, set_prepared_cache_size
+    w = make_problem(seed=92, q_lens=[700, 500], k_lens=[700, 900], hq=4, hk=2, d=64, qbs=64, kbs=64, keep=0.4, diag=True,
+                     causal=True, scale=None)
+    previous = set_prepared_cache_size(4)
+    calls = []
+    real = interface.hbsa_prepare
+    interface.hbsa_prepare = lambda *a, **k: calls.append(1) or real(*a, **k)
+    try:
+        ref = oracle_for(w)
+        for _ in range(3):
+            assert_close_to_oracle(_run(w), ref, "reused mask")
+        assert len(calls) == 1                                   # prepared once, reused twice
+        w.block_mask[:, :, 1] = ~w.block_mask[:, :, 1]           # in place: the version counter moves
+        assert_close_to_oracle(_run(w), oracle_for(w), "changed mask")
+        assert len(calls) == 2
+        with torch.cuda.stream(torch.cuda.Stream()):             # another stream gets its own workspace
+            torch.cuda.current_stream().wait_stream(torch.cuda.default_stream())
+            assert_close_to_oracle(_run(w), oracle_for(w), "other stream")
+        torch.cuda.synchronize()
+        assert len(calls) == 3
+        set_prepared_cache_size(0)                               # switched off: every call prepares
+        _run(w), _run(w)
+        assert len(calls) == 5
+    finally:
+        interface.hbsa_prepare = real
+        set_prepared_cache_size(previous)
+        interface.clear_prepared_cache()
+
+
 @pytest.mark.parametrize("d", [64, 128])
 def test_fp16_medium_problem(d):
     w = make_problem(seed=71, q_lens=[1500, 640], k_lens=[1500, 2048], hq=8, hk=4, d=d, qbs=128, kbs=64, keep=0.35, diag=True,
