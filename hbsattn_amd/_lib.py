@@ -37,6 +37,10 @@ def load() -> ctypes.CDLL:
         raise HBSAttnLibraryError(f"{LIB_PATH}: ABI version {lib.hbsa_abi_version()} != expected {ABI_VERSION}; rebuild")
     lib.hbsa_last_error.restype = ctypes.c_char_p
     lib.hbsa_last_error.argtypes = []
+    lib.hbsa_set_deterministic.restype = ctypes.c_int
+    lib.hbsa_set_deterministic.argtypes = [ctypes.c_int]
+    lib.hbsa_set_walk_min_bytes.restype = ctypes.c_longlong
+    lib.hbsa_set_walk_min_bytes.argtypes = [ctypes.c_longlong]
     lib.hbsa_fwd_workspace_bytes.restype = ctypes.c_size_t
     lib.hbsa_fwd_workspace_bytes.argtypes = [ctypes.c_int32] * 3
     lib.hbsa_fwd_workspace_bytes_dtype.restype = ctypes.c_size_t

@@ -30,6 +30,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <type_traits>
@@ -55,11 +56,12 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kThreads = 256;   // 4 wavefronts
 constexpr int kWaveRows = 32;   // query rows per wavefront (the MFMA N dimension)
 constexpr int kTileKeys = 64;   // keys per main-loop step
+constexpr int kWalkReportTiles = 8;   // an item adds its progress to its walk clock every so many tiles (a power of two)
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kMaxDevices = 64;            // devices of one process the launch caches cover
 constexpr float kLazyRescaleLog2 = 8.0f;  // running max may lag the true max by 2^8
 
-// Geometry of one q block, written by the pre-pass (32 bytes).
+// Geometry of one q block, written by the pre-pass (48 bytes).
 struct QBlockInfo {
   int32_t row_begin;   // token row of the block's first query
   int32_t rows;        // queries in the block (ragged last block of a sequence)
@@ -69,7 +71,10 @@ struct QBlockInfo {
   int32_t shift;       // k_len - q_len: bottom-right causal alignment
   int32_t nkblk;       // k blocks in the sequence
   int32_t kmax;        // exclusive in-sequence bound of keys any row of the block may see
+  int32_t seq;         // index of the sequence in the packed batch
+  int32_t pad[3];
 };
+static_assert(sizeof(QBlockInfo) == 48, "QBlockInfo is read as twelve 32-bit words");
 
 struct Sched;
 
@@ -80,6 +85,7 @@ struct PrepParams {
   QBlockInfo *info;
   uint32_t *bits;
   struct Sched *sched;
+  unsigned long long *clock;
   int32_t nqb, qbs, kbs, wpr, causal;
 };
 
@@ -116,6 +122,12 @@ struct FwdParams {
                   // the setup kernel derived them from the tensors' maxima
   int32_t nhead_k;
   struct Sched *sched;
+  // Walk order of the kept k blocks (see the kernel's comment).  walk != 0: the workgroups that work on
+  // one (kv head, sequence) keep near each other in key space through a shared clock, so that they find
+  // each other's K/V blocks in the L2; the summation order, and with it the last bits of the result,
+  // then depend on timing.  walk == 0: every item walks its blocks in ascending order (deterministic).
+  unsigned long long *clock;   // [nhead_k, num_q_block]: clock of (kv head, sequence index)
+  int32_t walk;
   float *lse;             // optional [total_q, nhead_q] log-sum-exp output (nullptr: none)
   int64_t lse_s, lse_h;   // its strides in elements
   // Split over key blocks (few, long work items): every (kv head, q block, slot group) becomes
@@ -153,8 +165,10 @@ __global__ __launch_bounds__(kThreads) void hbsa_prep_kernel(PrepParams p) {
     QBlockInfo r;
     r.row_begin = q0 + q_pos; r.rows = rows; r.key_begin = k0; r.klen = klen;
     r.q_pos = q_pos; r.shift = shift; r.nkblk = nkb; r.kmax = kmax;
+    r.seq = b; r.pad[0] = r.pad[1] = r.pad[2] = 0;
     p.info[g] = r;
   }
+  if (lane == 0) p.clock[(size_t)hk * p.nqb + g] = 0ull;   // the walk clocks start at zero (and every launch leaves them so)
   uint32_t *row = p.bits + ((size_t)hk * p.nqb + g) * p.wpr;
   const uint8_t *m = p.mask + hk * p.ms_h + g * p.ms_q + kb0 * p.ms_k;
   const int nw64 = (nkb + 63) >> 6;
@@ -330,7 +344,7 @@ __global__ __launch_bounds__(256) void hbsa_f32_stage_kernel(F32Tensor t, const 
 constexpr int kListCap = 1024;   // tile entries per list; longer items are expanded in chunks
 
 // Item header in LDS (16 ints).
-enum { H_HK = 0, H_QB, H_SUB, H_TOTAL, H_ROW_BEGIN, H_ROWS, H_KEY_BEGIN, H_Q_POS, H_SHIFT, H_PART, H_WORDS = 16 };
+enum { H_HK = 0, H_QB, H_SUB, H_TOTAL, H_ROW_BEGIN, H_ROWS, H_KEY_BEGIN, H_Q_POS, H_SHIFT, H_PART, H_T0, H_SEQ, H_NKBLK, H_WORDS = 16 };
 
 __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
@@ -485,6 +499,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   char *lds_k = lds;
   int *lds_hdr = (int *)(lds + 4 * TILE_BYTES);     // [2][H_WORDS]
   int *lds_list = lds_hdr + 2 * H_WORDS;            // [2][kListCap]
+  auto hdr_word = [&](int c_, int i) { return __builtin_amdgcn_readfirstlane(lds_hdr[c_ * H_WORDS + i]); };
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -560,7 +575,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
       claimed = (uint32_t)__builtin_amdgcn_readfirstlane((int)r);
     }
     if (st_hk >= 0) {
-      st_info = lane < 8 ? ((const uint32_t *)(p.info + st_qb))[lane] : 0u;
+      st_info = lane < 12 ? ((const uint32_t *)(p.info + st_qb))[lane] : 0u;
       st_bits = lane < p.wpr ? p.bits[(((size_t)st_part * p.nhead_k + st_hk) * p.nqb + st_qb) * p.wpr + lane] : 0u;
     }
   };
@@ -577,18 +592,110 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     }
     if (lane == 0) {
       hdr[H_HK] = st_hk; hdr[H_QB] = st_qb; hdr[H_SUB] = st_sub; hdr[H_TOTAL] = total; hdr[H_PART] = st_part;
+      hdr[H_T0] = 0;   // the item's walk starts at its first tile unless next_start() decides otherwise
     }
-    if (lane < 8) {   // QBlockInfo words: row_begin, rows, key_begin, klen, q_pos, shift, nkblk, kmax
+    if (lane < 9) {   // QBlockInfo words: row_begin, rows, key_begin, klen, q_pos, shift, nkblk, kmax, seq
       const int dst = lane == 0 ? H_ROW_BEGIN : lane == 1 ? H_ROWS : lane == 2 ? H_KEY_BEGIN : lane == 4 ? H_Q_POS
-                      : lane == 5 ? H_SHIFT : -1;
+                      : lane == 5 ? H_SHIFT : lane == 6 ? H_NKBLK : lane == 8 ? H_SEQ : -1;
       if (dst >= 0) hdr[dst] = (int)st_info;
     }
+  };
+
+  // ---- the walk clock (wavefront 0; p.walk != 0 only).  The online softmax does not care in which
+  // order an item's tiles are taken, and the workgroups that share an L2 (one XCD) work on items of
+  // one (kv head, sequence) at a time.  They keep near each other in key space, so that a K/V tile one
+  // of them fetched is still in the L2 when the others ask for it: every (kv head, sequence) has a
+  // clock word that holds, for the workgroups inside its items, their number (low 16 bits) and the sum
+  // of their positions (upper 48 bits; a position counts 64-key tiles of the sequence's key space and
+  // keeps growing over laps); one 64-bit atomic add updates both and returns both.  An item starts its
+  // walk at the first of its tiles at or after the clock's mean position, walks upwards, wraps to its
+  // first tile and ends where it began; it adds every step to the clock.  The start is decided two
+  // tiles before the item begins (its first tile is requested one tile before).
+  unsigned long long w_clk = 0;          // lane 0: the next item's clock as read three tiles before this item's end
+  unsigned long long *w_ptr = nullptr;   // this item's clock word, nullptr when it takes no part
+  int w_lap = 0, w_told = 0;             // the lap this item started in; the position its clock holds for it
+  int w_next_lap = 0;                    // lap the next item starts in (-1: it takes no part); the workgroup's
+                                         // first item finds the clocks empty: lap 0, first tile
+  int w_lt = 1;                          // 64-key tiles of this item's sequence (the length of a lap)
+  // what wavefront 0 remembers of the two items whose lists are in LDS (slot c_): clock word, lap length,
+  // and whether the item may take part (its tile list is a single chunk of at least three tiles)
+  unsigned long long *w_clock_of[2] = {nullptr, nullptr};
+  int w_tiles_of[2] = {1, 1};
+  bool w_part_of[2] = {false, false};
+  auto note_item = [&](int c_, int total_) {   // right after build(c_), from the staged records
+    const int nkblk = __builtin_amdgcn_readlane((int)st_info, 6);
+    const int seq = __builtin_amdgcn_readlane((int)st_info, 8);
+    w_part_of[c_] = p.walk != 0 && st_hk >= 0 && total_ >= 3 && total_ <= kListCap;
+    w_clock_of[c_] = p.clock + (size_t)(st_hk < 0 ? 0 : st_hk) * p.nqb + seq;
+    w_tiles_of[c_] = (nkblk * p.kbs + kTileKeys - 1) >> 6;
+  };
+  // three tiles before this item ends: read the next item's clock (a load that bypasses the CU's own
+  // cache; the clock words live in the XCD's L2, where the atomics on them are performed)
+  auto peek_next = [&](int cn) {
+    w_next_lap = -1;
+    if (!w_part_of[cn]) return;
+    if (lane == 0) w_clk = __hip_atomic_load(w_clock_of[cn], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    w_next_lap = 0;
+  };
+  // two tiles before it ends: the next item's start, from the clock's mean position
+  auto next_start = [&](int cn) {
+    if (w_next_lap < 0) return;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)w_clk);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(w_clk >> 32));
+    const uint32_t members = lo & 0xffffu;
+    if (members == 0) return;   // nobody there: start at the first tile, in lap 0
+    const float sum = (float)hi * 65536.f + (float)(lo >> 16);
+    int mean = __builtin_amdgcn_readfirstlane((int)(sum * __builtin_amdgcn_rcpf((float)members)));
+    const int lt = w_tiles_of[cn];
+    int lap = __builtin_amdgcn_readfirstlane((int)((float)mean * __builtin_amdgcn_rcpf((float)lt)));
+    int pos = mean - lap * lt;
+    while (pos < 0) { pos += lt; --lap; }
+    while (pos >= lt) { pos -= lt; ++lap; }
+    // entries of the (ascending) list below that position
+    const int n = hdr_word(cn, H_TOTAL);
+    int below = 0;
+    for (int i = 0; i < n; i += 64) {
+      const bool less = i + lane < n && (lds_list[cn * kListCap + i + lane] >> 8) < pos;   // entry >> 6 = key >> 4
+      below += __builtin_popcountll(__builtin_amdgcn_ballot_w64(less));
+    }
+    if (below >= n) {   // every tile of the item lies below: it starts the next lap at its first tile
+      below = 0;
+      ++lap;
+    }
+    if (lane == 0) lds_hdr[cn * H_WORDS + H_T0] = below;
+    w_next_lap = lap;
+  };
+  // first tile of an item: join its clock; later: add the progress since the last report (the atomics
+  // return nothing).  wraps: how often the walk has passed the end of the list (0 or 1).
+  auto report = [&](int c_, int kpos, bool first, int wraps) {
+    if (first) {
+      w_ptr = nullptr;
+      const int lap0 = w_next_lap;
+      w_next_lap = -1;   // the item after this one takes part only if peek_next() says so
+      if (lap0 < 0 || !w_part_of[c_]) return;
+      w_ptr = w_clock_of[c_];
+      w_lt = w_tiles_of[c_];
+      w_lap = lap0;
+      w_told = w_lap * w_lt + (kpos >> 6);
+      if (lane == 0) atomicAdd(w_ptr, ((unsigned long long)(uint32_t)w_told << 16) + 1ull);
+      return;
+    }
+    if (w_ptr == nullptr) return;
+    const int now = (w_lap + wraps) * w_lt + (kpos >> 6);
+    if (now != w_told && lane == 0) atomicAdd(w_ptr, (unsigned long long)(uint32_t)(now - w_told) << 16);
+    w_told = now;
+  };
+  auto leave_clock = [&]() {
+    if (w_ptr == nullptr) return;
+    if (lane == 0) atomicAdd(w_ptr, 0ull - (((unsigned long long)(uint32_t)w_told << 16) + 1ull));
+    w_ptr = nullptr;
   };
 
   if (wave == 0) {
     pending = claim();
     stage();
     build(0);
+    note_item(0, hdr_word(0, H_TOTAL));
     pending = claim();
     stage();
     pending = claim();
@@ -689,7 +796,6 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     }
   };
 
-  auto hdr_word = [&](int c, int i) { return __builtin_amdgcn_readfirstlane(lds_hdr[c * H_WORDS + i]); };
   // this wave's slice of an item: q head, first row inside the q block, rows
   auto q_row_ptr = [&](int hk, int sub, int row_begin, int rows, bool &act, int &hq, int &row0, int &nrows) {
     const int slot = sub * 4 + wave;
@@ -767,6 +873,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 
     if (wave == 0) {   // stay one item ahead: expand the staged item, stage the one after it
       build(c ^ 1);
+      if (p.walk) note_item(c ^ 1, hdr_word(c ^ 1, H_TOTAL));
       stage();
       pending = claim();
     }
@@ -791,27 +898,39 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 
     int nxt_hk = -1;          // known once the last tile is reached
     int chunk_base = 0;
+    // the walk starts at entry t0 of the (ascending) list and wraps: step t takes entry rot(t)
+    const int t0 = total <= kListCap ? hdr_word(c, H_T0) : 0;
     for (;;) {   // ---------------------------------------------------- chunks of the tile list (usually one)
       const int n = min(kListCap, total - chunk_base);
-      int held = 0;           // lane i: entry (window * 64 + i) of the current chunk
+      auto rot = [&](int x) { return x + t0 >= n ? x + t0 - n : x + t0; };   // x < n
+      int held = 0;           // lane i: entry of step (window * 64 + i) of the current chunk
       for (int t = 0; t < n; ++t) {   // ---------------------------------- one iteration per 64-key tile
-        if ((t & 63) == 0) held = (t + lane < n) ? lds_list[c * kListCap + t + lane] : 0;
+        if ((t & 63) == 0) held = (t + lane < n) ? lds_list[c * kListCap + rot(t + lane)] : 0;
         const int e = __builtin_amdgcn_readlane(held, t & 63);
         const int kpos = (e >> 6) << 4, valid = (e & 63) + 1;
 
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the current tile has landed in LDS
         // Everything fetched so far has arrived, the scheduler's records included: tell the
         // compiler here, or it waits for ALL outstanding memory traffic where they are first read.
-        asm volatile("" : "+v"(st_info), "+v"(st_bits), "+v"(pending));
+        asm volatile("" : "+v"(st_info), "+v"(st_bits), "+v"(pending), "+v"(w_clk));
         __syncthreads();                     // ... for every wave, and the other buffers are free
 
         const bool last = chunk_base + t + 1 == total;
+        // The clock is dealt with on few tiles only (wavefront 0; any work it does alone on every tile
+        // makes the other three wait at the next barrier): the item's first tile, every eighth, and
+        // the last three.
+        if (p.walk && wave == 0 && ((t & (kWalkReportTiles - 1)) == 0 || chunk_base + t + 3 >= total)) {
+          report(c, kpos, chunk_base + t == 0, t + t0 >= n ? 1 : 0);
+          if (chunk_base + t + 3 == total) peek_next(c ^ 1);
+          if (chunk_base + t + 2 == total) next_start(c ^ 1);
+          if (last) leave_clock();
+        }
         int nx_valid = 0;                 // > 0: a next tile exists and its loads go out during this tile
         const char *nx_vbase = nullptr, *nx_kbase = nullptr;
         if (t + 1 < n) {
           int e1;
           if (((t + 1) & 63) == 0) {
-            const int h1 = (t + 1 + lane < n) ? lds_list[c * kListCap + t + 1 + lane] : 0;
+            const int h1 = (t + 1 + lane < n) ? lds_list[c * kListCap + rot(t + 1 + lane)] : 0;
             e1 = __builtin_amdgcn_readlane(h1, 0);
           } else {
             e1 = __builtin_amdgcn_readlane(held, (t + 1) & 63);
@@ -823,7 +942,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         } else if (last) {
           nxt_hk = hdr_word(c ^ 1, H_HK);
           if (nxt_hk >= 0 && hdr_word(c ^ 1, H_TOTAL) > 0) {
-            const int e1 = __builtin_amdgcn_readfirstlane(lds_list[(c ^ 1) * kListCap]);
+            const int e1 = __builtin_amdgcn_readfirstlane(lds_list[(c ^ 1) * kListCap + hdr_word(c ^ 1, H_T0)]);
             const int tok = hdr_word(c ^ 1, H_KEY_BEGIN) + ((e1 >> 6) << 4);
             nx_valid = (e1 & 63) + 1;
             nx_vbase = tile_ptr(p.v + (int64_t)nxt_hk * p.v_h, tok, vs32);
@@ -1117,6 +1236,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     if (total == 0) {
       // No tile, hence no barrier since this item began: the next list may still be being written,
       // and nothing of the next item has been requested yet.
+      w_next_lap = -1;   // (nor has its walk been given a start: it takes no part in the clock)
       __builtin_amdgcn_s_waitcnt(0x0F70);   // keeps "every fetch has arrived" true on every path
       __syncthreads();
       nxt_hk = hdr_word(c ^ 1, H_HK);
@@ -1208,9 +1328,24 @@ int fail(int code, const char *fmt, ...) {
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 inline int words_per_row(int num_k_block) { return 2 * ((num_k_block + 63) / 64); }
-// workspace layout: QBlockInfo[num_q_block] | Sched | bit words
+// workspace layout: QBlockInfo[num_q_block] | Sched | walk clocks [nhead_k, num_q_block] | bit words
 inline size_t sched_offset(int num_q_block) { return align_up((size_t)num_q_block * sizeof(QBlockInfo), 256); }
-inline size_t bits_offset(int num_q_block) { return sched_offset(num_q_block) + align_up(sizeof(Sched), 256); }
+inline size_t clock_offset(int num_q_block) { return sched_offset(num_q_block) + align_up(sizeof(Sched), 256); }
+inline size_t bits_offset(int nhead_k, int num_q_block) {
+  return clock_offset(num_q_block) + align_up((size_t)nhead_k * num_q_block * sizeof(unsigned long long), 256);
+}
+
+// Deterministic mode: every item walks its tiles in ascending order, so results are bitwise
+// reproducible; otherwise very large problems use the clocked walk (results then vary in their last
+// bits from run to run).  Initial value from the environment variable HBSATTN_AMD_DETERMINISTIC.
+int g_deterministic = [] {
+  const char *e = std::getenv("HBSATTN_AMD_DETERMINISTIC");
+  return e != nullptr && e[0] != 0 && e[0] != '0' ? 1 : 0;
+}();
+// K + V bytes of one kv head from which the clocked walk is used.  Measured on MI355X: at 64K-token
+// sequences with 30 % of the blocks kept the walk takes a seventh off the HBM traffic and 5 % off the
+// time; at 32K tokens and 10 % kept it takes 6 % off the traffic and nothing off the time.
+long long g_walk_min_bytes = 192ll << 20;
 
 // rows must be 16-byte aligned: strides (in elements) multiples of 8 for 16-bit types, of 4 for fp32
 int check_strides(const int64_t *strides, bool f32) {
@@ -1515,6 +1650,18 @@ extern "C" {
 
 int hbsa_abi_version(void) { return HBSA_ABI_VERSION; }
 
+int hbsa_set_deterministic(int on) {
+  const int previous = g_deterministic;
+  g_deterministic = on ? 1 : 0;
+  return previous;
+}
+
+long long hbsa_set_walk_min_bytes(long long bytes) {
+  const long long previous = g_walk_min_bytes;
+  if (bytes >= 0) g_walk_min_bytes = bytes;
+  return previous;
+}
+
 const char *hbsa_last_error(void) { return g_err; }
 
 int hbsa_calculate_blocks(const int32_t *cu_seqlen, int32_t batch, int32_t block_size, int32_t *num_block,
@@ -1547,7 +1694,7 @@ int hbsa_calculate_blocks(const int32_t *cu_seqlen, int32_t batch, int32_t block
 size_t hbsa_fwd_workspace_bytes(int32_t nhead_k, int32_t num_q_block, int32_t num_k_block) {
   if (nhead_k <= 0 || num_q_block <= 0 || num_k_block <= 0) return 256;
   const size_t bits = align_up((size_t)nhead_k * num_q_block * words_per_row(num_k_block) * sizeof(uint32_t), 256);
-  return bits_offset(num_q_block) + bits;
+  return bits_offset(nhead_k, num_q_block) + bits;
 }
 
 size_t hbsa_fwd_workspace_bytes_dtype(int32_t dtype, int32_t total_q, int32_t total_k, int32_t nhead_q,
@@ -1594,8 +1741,9 @@ int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens, c
   pp.cu_num_q_block = cu_num_q_block; pp.cu_num_k_block = cu_num_k_block;
   pp.mask = block_mask; pp.ms_h = mask_strides[0]; pp.ms_q = mask_strides[1]; pp.ms_k = mask_strides[2];
   pp.info = (QBlockInfo *)workspace;
-  pp.bits = (uint32_t *)((char *)workspace + bits_offset(num_q_block));
+  pp.bits = (uint32_t *)((char *)workspace + bits_offset(nhead_k, num_q_block));
   pp.sched = (Sched *)((char *)workspace + sched_offset(num_q_block));
+  pp.clock = (unsigned long long *)((char *)workspace + clock_offset(num_q_block));
   pp.nqb = num_q_block; pp.qbs = q_block_size; pp.kbs = k_block_size; pp.wpr = words_per_row(num_k_block);
   pp.causal = causal ? 1 : 0;
   hipLaunchKernelGGL(hbsa_prep_kernel, dim3((num_q_block + 3) / 4, nhead_k), dim3(kThreads), 0, (hipStream_t)stream, pp);
@@ -1650,8 +1798,9 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
   FwdParams fp;
   fp.q = (const char *)q; fp.k = (const char *)k; fp.v = (const char *)v; fp.out = (char *)out;
   fp.info = (const QBlockInfo *)workspace;
-  fp.bits = (const uint32_t *)((const char *)workspace + bits_offset(num_q_block));
+  fp.bits = (const uint32_t *)((const char *)workspace + bits_offset(nhead_k, num_q_block));
   fp.sched = (Sched *)((char *)workspace + sched_offset(num_q_block));
+  fp.clock = (unsigned long long *)((char *)workspace + clock_offset(num_q_block));
   fp.nhead_k = nhead_k;
   fp.f32 = f32 ? 1 : 0;
   fp.lse = lse;
@@ -1703,6 +1852,9 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
       fp.nparts = parts;
   }
   fp.div_nparts = make_fast_div((uint32_t)fp.nparts);
+  // the clocked walk: block sizes that are whole tiles, work that is not split, K/V of a head beyond what an L2 holds
+  fp.walk = (!g_deterministic && fp.nparts == 1 && k_block_size % kTileKeys == 0 &&
+             2ll * total_k * headdim * 2 >= g_walk_min_bytes) ? 1 : 0;
 
   if (f32_exact) {
     const float c_signed = softmax_scale * kLog2e;
@@ -1868,7 +2020,7 @@ int hbsa_bwd(const void *q, const void *k, const void *v, const void *out, const
   bp.dq = (char *)dq; bp.dk = (char *)dk; bp.dv = (char *)dv;
   bp.lse = lse; bp.delta = (const float *)bwd_workspace;
   bp.info = (const QBlockInfo *)workspace;
-  bp.bits = (const uint32_t *)((const char *)workspace + bits_offset(num_q_block));
+  bp.bits = (const uint32_t *)((const char *)workspace + bits_offset(nhead_k, num_q_block));
   bp.cu_k = cu_k_seqlens; bp.cu_num_q_block = cu_num_q_block; bp.cu_num_k_block = cu_num_k_block;
   bp.q_s = strides[0] * es; bp.q_h = strides[1] * es; bp.k_s = strides[2] * es; bp.k_h = strides[3] * es;
   bp.v_s = strides[4] * es; bp.v_h = strides[5] * es; bp.do_s = strides[8] * es; bp.do_h = strides[9] * es;

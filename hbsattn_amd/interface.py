@@ -41,6 +41,15 @@ def set_fp32_mode(mode: str) -> str:
     return previous
 
 
+def set_deterministic(on: bool) -> bool:
+    """Deterministic mode of the library (``hbsa_set_deterministic``): with it on every query block walks
+    its key tiles in ascending order and results are bitwise reproducible at every size; with it off
+    (the default unless HBSATTN_AMD_DETERMINISTIC is set) very large problems order the walk by a clock
+    shared between workgroups, which saves HBM traffic and lets the last bits of the result depend on
+    timing.  Returns the previous setting."""
+    return bool(_lib.load().hbsa_set_deterministic(1 if on else 0))
+
+
 def _dtype_code(dtype: torch.dtype) -> int:
     if dtype == torch.float32 and _fp32_mode == "fast":
         return _lib.DTYPE_F32_STAGED16

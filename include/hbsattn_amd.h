@@ -49,6 +49,26 @@ int hbsa_abi_version(void);
 const char *hbsa_last_error(void);
 
 /*
+ * Deterministic mode (process-wide; returns the previous setting; initial value 1 if the environment
+ * variable HBSATTN_AMD_DETERMINISTIC is set to something other than 0, else 0).  The attention kernel
+ * may visit the kept key tiles of a query block in any order.  With the mode off, problems whose K and
+ * V of one kv head reach hbsa_set_walk_min_bytes (192 MiB unless changed; k_block_size a multiple of 64)
+ * start every query block's walk at the mean position of the workgroups that are inside the same
+ * (kv head, sequence), kept in a clock word per (kv head, sequence) in the workspace, and wrap around:
+ * those workgroups share an L2, and the K/V tiles one of them fetched are then found there by the
+ * others.  The fp32 summation order then depends on timing and results differ from run to run in their
+ * last bits (the error against an exact evaluation is unchanged).  With the mode on, and for smaller
+ * problems, every query block walks its tiles in ascending order and results are bitwise reproducible.
+ * The reference's kernels always walk in ascending order (reference
+ * hbsattn/fwd_triton_auto_tile_size.py:153-164).
+ */
+int hbsa_set_deterministic(int on);
+
+/* Size (K + V bytes of one kv head) from which the clocked walk above is used; a negative value only
+ * reads the setting.  Returns the previous value. */
+long long hbsa_set_walk_min_bytes(long long bytes);
+
+/*
  * Block geometry of a packed variable-length batch, on the HOST (all pointers are host memory):
  * the counterpart of hbsattn.utils.calculate_blocks (reference hbsattn/utils.py:7-50) for callers
  * without torch.  Blocks restart at every sequence start and the last block of a sequence may be

@@ -469,6 +469,41 @@ def test_attention_launches_leave_the_work_queues_ready_for_the_next_launch():
         assert torch.equal(out4, first4), f"launch {i}, 4 q heads"
 
 
+@pytest.mark.parametrize("causal,kbs,qbs", [(True, 128, 128), (False, 64, 64), (True, 192, 64)])
+def test_clocked_walk_matches_the_oracle_and_leaves_its_clocks_at_zero(causal, kbs, qbs):
+    """The walk order used for very large problems (an item starts at the mean position of the workgroups
+    inside the same kv head and sequence, and wraps), forced on here by a zero size threshold: the
+    result is within the forward's tolerance of the oracle and, from launch to launch, equal up to the
+    summation order; every launch leaves the clock words of the workspace at zero."""
+    from hbsattn_amd import _lib
+    from hbsattn_amd.interface import hbsa_prepare, hbsa_run
+    lib = _lib.load()
+    w = make_problem(seed=93, q_lens=[4096, 1536, 2048], k_lens=[4096, 3000, 2048], hq=16, hk=16, d=128, qbs=qbs, kbs=kbs,
+                     keep=0.25, diag=True, causal=causal, scale=None)
+    ref = oracle_for(w)
+    straight = _run(w)                                      # ascending walk (the problem is far below the threshold)
+    previous = lib.hbsa_set_walk_min_bytes(0)
+    try:
+        assert not lib.hbsa_set_deterministic(0)
+        prepared = hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, qbs, kbs, causal, w.q_meta[0], w.q_meta[2],
+                                w.q_meta[3], w.k_meta[0], w.k_meta[3])
+        nqb, nhk = w.q_meta[0], w.k.shape[1]
+        clock_at = (nqb * 48 + 255) // 256 * 256 + 256       # geometry records, then the 256-byte launch record
+        clocks = prepared.workspace[clock_at:clock_at + 8 * nhk * nqb].view(torch.int64)
+        for launch in range(3):
+            out = hbsa_run(w.q, w.k, w.v, prepared, None)
+            torch.cuda.synchronize()
+            assert_close_to_oracle(out, ref, f"clocked walk, launch {launch}")
+            assert (out.float() - straight.float()).abs().max().item() <= 2e-2
+            assert int(clocks.abs().max()) == 0, "a workgroup left its position in a clock word"
+        # deterministic mode overrides the threshold: bitwise equal to the ascending walk
+        lib.hbsa_set_deterministic(1)
+        assert torch.equal(hbsa_run(w.q, w.k, w.v, prepared, None), straight)
+    finally:
+        lib.hbsa_set_deterministic(0)
+        lib.hbsa_set_walk_min_bytes(previous)
+
+
 def test_prepared_masks_are_reused_only_for_unchanged_tensors():
     from hbsattn_amd import interface, set_prepared_cache_size
     w = make_problem(seed=92, q_lens=[700, 500], k_lens=[700, 900], hq=4, hk=2, d=64, qbs=64, kbs=64, keep=0.4, diag=True,
