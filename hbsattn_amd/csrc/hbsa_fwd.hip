@@ -113,7 +113,8 @@ struct FwdParams {
   int64_t q_s, q_h, k_s, k_h, v_s, v_h, o_s, o_h;  // bytes
   int32_t nqb, ratio, kbs, wpr, causal;
   int32_t wps;    // wave slots per q head = ceil(q_block_size / 32)
-  int32_t nsub;   // workgroups per (kv head, q block) = ceil(ratio * wps / 4)
+  int32_t nw;     // wavefronts per workgroup (4 or 8)
+  int32_t nsub;   // workgroups per (kv head, q block) = ceil(ratio * wps / nw)
   uint32_t q_sign;  // 0x80008000 when softmax_scale < 0 (Q is negated, |scale| used)
   float c;        // |softmax_scale| * log2(e)
   float lag;      // kLazyRescaleLog2 / c: how far the running max may lag, in raw score units
@@ -484,14 +485,18 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-template <int D, typename E, bool OUT32>
-__global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
+template <int D, typename E, bool OUT32, int NW>
+__global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) {
   // OUT32: fp32 output (the fp32-input path; q/k/v are then fp16 staging copies)
+  // NW: wavefronts (wave slots) of a workgroup, 4 or 8.  Eight are used when the q heads of a GQA group
+  // and the 32-row slices of a q block give an item more than four wave slots: one workgroup per CU then
+  // stages every K/V tile once for all of them instead of two workgroups staging it each.
   constexpr int RB = D * 2;            // row bytes
   constexpr int CPR = RB / 16;         // 16-byte chunks per row
   constexpr int RPG = 16 / CPR > 0 ? 16 / CPR : 1;  // rows per 256-byte bank sweep
   constexpr int TILE_BYTES = kTileKeys * RB;
-  constexpr int LOADS = CPR / 4;       // 16-byte loads per thread per tile per operand
+  constexpr int LOADS = CPR / NW;      // 16-byte loads per thread per tile per operand
+  static_assert(LOADS >= 1, "a tile row has fewer 16-byte chunks than the workgroup has wavefronts");
   constexpr int KSTEPS = D / 16;       // MFMA k-steps of Q.K^T
   constexpr int DT = D / 32;           // 32-row tiles of O^T
 
@@ -707,7 +712,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   uint32_t ld_koff[LOADS], ld_voff[LOADS];   // byte offset of the thread's chunk from the tile's first row
   const uint32_t ks32 = (uint32_t)p.k_s, vs32 = (uint32_t)p.v_s;   // row strides in bytes (the host checks they fit)
   auto ld_place = [&](int i, int &r, uint32_t &kchunk, uint32_t &vchunk) {
-    const int c = (i * 4 + wave) * 64 + lane;
+    const int c = (i * NW + wave) * 64 + lane;
     const int pc = c % CPR;
     r = c / CPR;
     kchunk = (uint32_t)((pc ^ ((r / RPG) % CPR)) * 16);
@@ -742,7 +747,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
     if (valid == kTileKeys) {
       static_for<0, LOADS>([&](auto i_) {
         constexpr int i = decltype(i_)::value;
-        dma16(std::integral_constant<int, lds_off + i * 4096>{}, base, V_PART ? ld_voff[i] : ld_koff[i], l0);
+        dma16(std::integral_constant<int, lds_off + i * NW * 1024>{}, base, V_PART ? ld_voff[i] : ld_koff[i], l0);
       });
     } else {   // ragged tail of a run: rows past the end re-read the last valid row (masked later)
       static_for<0, LOADS>([&](auto i_) {
@@ -750,7 +755,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
         int r; uint32_t kc, vc;
         ld_place(i, r, kc, vc);
         r = min(r, valid - 1);
-        dma16(std::integral_constant<int, lds_off + i * 4096>{}, base, (uint32_t)r * (V_PART ? vs32 : ks32) + (V_PART ? vc : kc), l0);
+        dma16(std::integral_constant<int, lds_off + i * NW * 1024>{}, base, (uint32_t)r * (V_PART ? vs32 : ks32) + (V_PART ? vc : kc), l0);
       });
     }
   };
@@ -798,7 +803,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
 
   // this wave's slice of an item: q head, first row inside the q block, rows
   auto q_row_ptr = [&](int hk, int sub, int row_begin, int rows, bool &act, int &hq, int &row0, int &nrows) {
-    const int slot = sub * 4 + wave;
+    const int slot = sub * NW + wave;
     const int head_in_group = slot / p.wps;
     row0 = (slot % p.wps) * kWaveRows;
     nrows = min(kWaveRows, rows - row0);
@@ -816,7 +821,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_kernel(FwdParams p) {
   // (v_permlane16_swap), which leaves k-step 2k in A_k and k-step 2k+1 in B_k.
   short8v qf[KSTEPS];
   auto load_q = [&](int hk, int sub, int row_begin, int rows) {
-    const int slot = sub * 4 + wave;
+    const int slot = sub * NW + wave;
     const int head_in_group = slot / p.wps;
     const int row0 = (slot % p.wps) * kWaveRows;
     if (head_in_group >= p.ratio || rows - row0 <= 0) return;   // this wavefront has no rows: qf is never used
@@ -1374,6 +1379,11 @@ F32Tensor f32_tensor(int i, const void *q, const void *k, const void *v, const i
   return {(const float *)x, strides[2 * i], strides[2 * i + 1], heads, dshift, tokens * heads * headdim / 4};
 }
 
+// Wavefronts per workgroup of the 16-bit attention kernel for an item of `slots` wave slots (32-row
+// slices of a q block x q heads of a GQA group): eight when the item has more than four slots, so that
+// one workgroup stages its K/V tiles once (head dims from 64; the fp32 kernel always has four).
+inline int fwd_wavefronts(int slots, int headdim, bool f32_exact) { return (!f32_exact && slots > 4 && headdim >= 64) ? 8 : 4; }
+
 // Split over key blocks pays when the work items cannot fill the device: fewer than one per CU.
 // Returns the number of parts (1 = no split) for the current device.
 int split_parts(long long items, int num_k_block) {
@@ -1401,20 +1411,20 @@ inline size_t split_bytes(int parts, int total_q, int nhead_q, int nhead_k, int 
          align_up((size_t)parts * total_q * nhead_q * 4, 256);
 }
 
-int persistent_grid(const void *kernel, int lds_bytes) {
+int persistent_grid(const void *kernel, int lds_bytes, int threads) {
   int dev = 0, cus = 0, per_cu = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kThreads, lds_bytes) != hipSuccess) return 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, lds_bytes) != hipSuccess) return 0;
   if (per_cu < 1) return 0;
   if (per_cu > 4) per_cu = 4;
   return cus * per_cu;
 }
 
-template <int D, typename E, bool OUT32>
-int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
+template <int D, typename E, bool OUT32, int NW>
+int launch_fwd_nw(const FwdParams &fp, long long items, hipStream_t stream) {
   constexpr int lds_bytes = 4 * kTileKeys * D * 2 + 2 * H_WORDS * 4 + 2 * kListCap * 4;
-  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E, OUT32>);
+  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E, OUT32, NW>);
   // workgroups that fit the current device at once; the attribute and the occupancy are per device
   static thread_local int resident_of[kMaxDevices] = {};
   int dev = 0;
@@ -1424,14 +1434,21 @@ int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
   if (resident == 0) {
     hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    resident = persistent_grid(kernel, lds_bytes);
+    resident = persistent_grid(kernel, lds_bytes, NW * 64);
     if (resident <= 0) return fail(HBSA_ERR_UNSUPPORTED, "could not size the persistent grid");
   }
   const int grid = (int)(items < resident ? items : resident);
-  hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32>), dim3(grid), dim3(kThreads), lds_bytes, stream, fp);
+  hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32, NW>), dim3(grid), dim3(NW * 64), lds_bytes, stream, fp);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail((int)e, "hbsa_fwd_kernel launch: %s", hipGetErrorString(e));
   return 0;
+}
+template <int D, typename E, bool OUT32>
+int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
+  if constexpr (D >= 64) {
+    if (fp.nw == 8) return launch_fwd_nw<D, E, OUT32, 8>(fp, items, stream);
+  }
+  return launch_fwd_nw<D, E, OUT32, 4>(fp, items, stream);
 }
 
 
@@ -1710,7 +1727,8 @@ size_t hbsa_fwd_split_workspace_bytes(int32_t total_q, int32_t nhead_q, int32_t 
   if (total_q <= 0 || nhead_q <= 0 || nhead_k <= 0 || headdim <= 0 || num_q_block <= 0 || num_k_block <= 0 || q_block_size <= 0)
     return 0;
   const int ratio = nhead_q / nhead_k, wps = (q_block_size + kWaveRows - 1) / kWaveRows;
-  const long long items = (long long)nhead_k * num_q_block * ((ratio * wps + 3) / 4);
+  const int nw = fwd_wavefronts(ratio * wps, headdim, false);
+  const long long items = (long long)nhead_k * num_q_block * ((ratio * wps + nw - 1) / nw);
   return split_bytes(split_parts(items, num_k_block), total_q, nhead_q, nhead_k, headdim, num_q_block, num_k_block);
 }
 
@@ -1830,7 +1848,8 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
   fp.nqb = num_q_block; fp.ratio = nhead_q / nhead_k; fp.kbs = k_block_size; fp.wpr = words_per_row(num_k_block);
   fp.causal = causal ? 1 : 0;
   fp.wps = (q_block_size + kWaveRows - 1) / kWaveRows;
-  fp.nsub = (fp.ratio * fp.wps + 3) / 4;
+  fp.nw = fwd_wavefronts(fp.ratio * fp.wps, headdim, f32_exact);
+  fp.nsub = (fp.ratio * fp.wps + fp.nw - 1) / fp.nw;
   fp.div_nsub = make_fast_div((uint32_t)fp.nsub);
   fp.div_nqb = make_fast_div((uint32_t)num_q_block);
   fp.div_kbs = make_fast_div((uint32_t)k_block_size);

@@ -153,7 +153,8 @@ def test_full_size_properties_config2():
 
 def test_gqa_equals_mha_on_repeated_kv_bitwise():
     # (enough work items that neither call is split over key blocks: the two would split differently)
-    w = make_problem(seed=11, q_lens=[3000, 4100], k_lens=[3000, 4100], hq=8, hk=2, d=128, qbs=64, kbs=128, keep=0.4,
+    # (the GQA call runs workgroups of eight wavefronts, one per kv head and q block: 2 x 223 items)
+    w = make_problem(seed=11, q_lens=[6000, 8200], k_lens=[6000, 8200], hq=8, hk=2, d=128, qbs=64, kbs=128, keep=0.4,
                      diag=True, causal=True, scale=None)
     out = _run(w)
     k_rep, v_rep = w.k.repeat_interleave(4, 1), w.v.repeat_interleave(4, 1)
