@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhbsattn_amd.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 DTYPE_BF16 = 0
 DTYPE_F16 = 1
@@ -53,7 +53,7 @@ def load() -> ctypes.CDLL:
     lib.hbsa_fwd_static.restype = ctypes.c_int
     lib.hbsa_fwd_static.argtypes = [vp] * 10 + [ctypes.c_int32] * 12 + [ctypes.c_float, i64p, vp]
     lib.hbsa_fwd_prepare.restype = ctypes.c_int
-    lib.hbsa_fwd_prepare.argtypes = [vp] * 7 + [ctypes.c_size_t] + [ctypes.c_int32] * 7 + [i64p, vp]
+    lib.hbsa_fwd_prepare.argtypes = [vp] * 7 + [ctypes.c_size_t] + [ctypes.c_int32] * 9 + [i64p, vp]
     lib.hbsa_fwd_run.restype = ctypes.c_int
     lib.hbsa_fwd_run.argtypes = [vp] * 5 + [ctypes.c_size_t] + [ctypes.c_int32] * 11 + [ctypes.c_float, i64p, vp]
     lib.hbsa_fwd_run_lse.restype = ctypes.c_int

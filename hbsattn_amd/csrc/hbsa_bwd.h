@@ -202,6 +202,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   const int qb_rev = bx / p.nsub, sub = bx - qb_rev * p.nsub;
   const int qb = p.nqb - 1 - qb_rev;
   const QBlockInfo inf = p.info[qb];
+  if (inf.rows <= 0) return;   // a q block of a sequence the pre-pass skipped (boundaries outside the tensors)
 
   const int slot = sub * 4 + wave;
   const int head_in_group = slot / p.wps;
@@ -327,6 +328,10 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
 
   int b = 0;   // the sequence the k block belongs to
   while (b + 1 < p.batch && p.cu_num_k_block[b + 1] <= kb) ++b;
+  {   // a sequence the pre-pass skipped (boundaries outside the tensors) has empty q block records: nothing to do
+    const int first_qb = p.cu_num_q_block[b];
+    if (first_qb < 0 || first_qb >= p.nqb || (first_qb < p.cu_num_q_block[b + 1] && p.info[first_qb].rows <= 0)) return;
+  }
   const int kbl = kb - p.cu_num_k_block[b];          // in-sequence index of the k block
   const int k0 = p.cu_k[b], klen = p.cu_k[b + 1] - k0;
   const int krows = min(p.kbs, klen - kbl * p.kbs);  // keys in the block
@@ -522,6 +527,10 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
 
   int b = 0;   // the sequence the k block belongs to
   while (b + 1 < p.batch && p.cu_num_k_block[b + 1] <= kb) ++b;
+  {   // a sequence the pre-pass skipped (boundaries outside the tensors) has empty q block records: nothing to do
+    const int first_qb = p.cu_num_q_block[b];
+    if (first_qb < 0 || first_qb >= p.nqb || (first_qb < p.cu_num_q_block[b + 1] && p.info[first_qb].rows <= 0)) return;
+  }
   const int kbl = kb - p.cu_num_k_block[b];
   const int k0 = p.cu_k[b], klen = p.cu_k[b + 1] - k0;
   const int krows = min(p.kbs, klen - kbl * p.kbs);

@@ -87,6 +87,7 @@ struct PrepParams {
   struct Sched *sched;
   unsigned long long *clock;
   int32_t nqb, qbs, kbs, wpr, causal;
+  int32_t batch, nkb, total_q, total_k;   // bounds the sequences' boundaries are checked against
 };
 
 // Division by a launch constant d, exact for 0 <= n < 2^31: n / d == (n * m) >> s with
@@ -152,21 +153,31 @@ __global__ __launch_bounds__(kThreads) void hbsa_prep_kernel(PrepParams p) {
   if (g >= p.nqb) return;
   const int hk = blockIdx.y;
   const int b = p.q_block_to_batch[g];
-  const int q0 = p.cu_q[b], qlen = p.cu_q[b + 1] - q0;
-  const int k0 = p.cu_k[b], klen = p.cu_k[b + 1] - k0;
-  const int q_pos = (g - p.cu_num_q_block[b]) * p.qbs;
-  const int rows = min(p.qbs, qlen - q_pos);
+  // A sequence whose boundaries do not fit the tensors and the block counts (a wrong cu_seqlens, q/k/v
+  // shorter than it says) is skipped as a whole: its q blocks get empty records and bit rows, which
+  // every kernel that reads them treats as "nothing to do", so nothing outside the tensors is touched.
+  bool ok = b >= 0 && b < p.batch;
+  int q0 = 0, qlen = 0, k0 = 0, klen = 0, kb0 = 0, nkb = 0, q_pos = 0;
+  if (ok) {
+    q0 = p.cu_q[b]; qlen = p.cu_q[b + 1] - q0;
+    k0 = p.cu_k[b]; klen = p.cu_k[b + 1] - k0;
+    kb0 = p.cu_num_k_block[b]; nkb = p.cu_num_k_block[b + 1] - kb0;
+    const int qb0 = p.cu_num_q_block[b];
+    q_pos = (g - qb0) * p.qbs;
+    ok = q0 >= 0 && qlen > 0 && (int64_t)q0 + qlen <= p.total_q && k0 >= 0 && klen >= 0 && (int64_t)k0 + klen <= p.total_k &&
+         kb0 >= 0 && nkb >= 0 && (int64_t)kb0 + nkb <= p.nkb && (int64_t)nkb * p.kbs >= klen && g >= qb0 && q_pos < qlen;
+  }
+  if (!ok) { q0 = qlen = k0 = klen = kb0 = nkb = q_pos = 0; }
+  const int rows = ok ? min(p.qbs, qlen - q_pos) : 0;
   const int shift = klen - qlen;
-  const int kb0 = p.cu_num_k_block[b];
-  const int nkb = p.cu_num_k_block[b + 1] - kb0;
   int kmax = p.causal ? min(klen, q_pos + rows + shift) : klen;
-  if (kmax < 0) kmax = 0;
+  if (kmax < 0 || !ok) kmax = 0;
   const int nvis = min(nkb, (kmax + p.kbs - 1) / p.kbs);
   if (hk == 0 && lane == 0) {
     QBlockInfo r;
     r.row_begin = q0 + q_pos; r.rows = rows; r.key_begin = k0; r.klen = klen;
     r.q_pos = q_pos; r.shift = shift; r.nkblk = nkb; r.kmax = kmax;
-    r.seq = b; r.pad[0] = r.pad[1] = r.pad[2] = 0;
+    r.seq = ok ? b : 0; r.pad[0] = r.pad[1] = r.pad[2] = 0;
     p.info[g] = r;
   }
   if (lane == 0) p.clock[(size_t)hk * p.nqb + g] = 0ull;   // the walk clocks start at zero (and every launch leaves them so)
@@ -1736,9 +1747,10 @@ int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens, c
                      const int32_t *q_block_to_batch, const int32_t *cu_num_q_block, const int32_t *cu_num_k_block,
                      void *workspace, size_t workspace_bytes, int32_t batch, int32_t nhead_k, int32_t num_q_block,
                      int32_t num_k_block, int32_t q_block_size, int32_t k_block_size, int32_t causal,
-                     const int64_t *mask_strides, void *stream) {
+                     int32_t total_q, int32_t total_k, const int64_t *mask_strides, void *stream) {
   g_err[0] = 0;
-  if (batch < 0 || num_q_block < 0 || num_k_block < 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "negative size");
+  if (batch < 0 || num_q_block < 0 || num_k_block < 0 || total_q < 0 || total_k < 0)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "negative size");
   if (num_q_block == 0) return 0;
   if (!cu_q_seqlens || !cu_k_seqlens || !block_mask || !q_block_to_batch || !cu_num_q_block || !cu_num_k_block ||
       !workspace || !mask_strides)
@@ -1764,6 +1776,7 @@ int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens, c
   pp.clock = (unsigned long long *)((char *)workspace + clock_offset(num_q_block));
   pp.nqb = num_q_block; pp.qbs = q_block_size; pp.kbs = k_block_size; pp.wpr = words_per_row(num_k_block);
   pp.causal = causal ? 1 : 0;
+  pp.batch = batch; pp.nkb = num_k_block; pp.total_q = total_q; pp.total_k = total_k;
   hipLaunchKernelGGL(hbsa_prep_kernel, dim3((num_q_block + 3) / 4, nhead_k), dim3(kThreads), 0, (hipStream_t)stream, pp);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail((int)e, "hbsa_prep_kernel launch: %s", hipGetErrorString(e));
@@ -1940,7 +1953,7 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32
   }
   int rc = hbsa_fwd_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_to_batch, cu_num_q_block, cu_num_k_block,
                             workspace, workspace_bytes, batch, nhead_k, num_q_block, num_k_block, q_block_size,
-                            k_block_size, causal, strides + 8, stream);
+                            k_block_size, causal, total_q, total_k, strides + 8, stream);
   if (rc != 0) return rc;
   return hbsa_fwd_run(q, k, v, out, workspace, workspace_bytes, dtype, total_q, total_k, nhead_q, nhead_k, headdim,
                       num_q_block, num_k_block, q_block_size, k_block_size, causal, softmax_scale, strides, stream);

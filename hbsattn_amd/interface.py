@@ -138,7 +138,9 @@ def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_s
                  q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, run_shape=None) -> PreparedMask:
     """Runs the pre-pass kernel (``hbsa_fwd_prepare``) on the current stream.  ``run_shape`` =
     ``(dtype, total_q, total_k, nhead_q, headdim)`` of the q/k/v the mask will be used with sizes the
-    workspace for them at once (``hbsa_run`` grows it otherwise)."""
+    workspace for them at once (``hbsa_run`` grows it otherwise) and gives the pre-pass the token counts it
+    checks the sequence boundaries against: a sequence that does not fit the tensors is skipped as a
+    whole instead of being read and written out of bounds (without ``run_shape`` nothing is checked)."""
     if not block_mask.is_cuda:
         raise RuntimeError("hbsattn_amd runs on MI355X only: block_mask must be a CUDA(HIP) tensor; there is no CPU path")
     _check_block_sizes(q_block_size, k_block_size)
@@ -157,8 +159,10 @@ def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_s
     lib = _lib.load()
     nhead_k = block_mask.shape[0]
     ws_bytes = int(lib.hbsa_fwd_workspace_bytes(nhead_k, num_q_block, num_k_block))
+    bound_q = bound_k = 2 ** 31 - 1
     if run_shape is not None:
         dtype, total_q, total_k, nhead_q, headdim = run_shape
+        bound_q, bound_k = int(total_q), int(total_k)
         d_run = next((d for d in _NATIVE_HEADDIMS if d >= headdim), headdim)
         if dtype in _DTYPE_CODES and total_q > 0 and nhead_q > 0:
             ws_bytes = max(ws_bytes, _run_workspace_bytes(lib, dev, _dtype_code(dtype), total_q, total_k, nhead_q, nhead_k,
@@ -170,8 +174,8 @@ def hbsa_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_s
     with torch.cuda.device(dev):
         rc = lib.hbsa_fwd_prepare(cu_q.data_ptr(), cu_k.data_ptr(), block_mask.data_ptr(), qb2b.data_ptr(),
                                   cu_nqb.data_ptr(), cu_nkb.data_ptr(), workspace.data_ptr(), ws_bytes, cu_q.numel() - 1,
-                                  nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, int(bool(causal)), mstr,
-                                  torch.cuda.current_stream().cuda_stream)
+                                  nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, int(bool(causal)),
+                                  bound_q, bound_k, mstr, torch.cuda.current_stream().cuda_stream)
     if rc != 0:
         raise RuntimeError(f"hbsa_fwd_prepare failed (code {rc}): {_lib.last_error()}")
     return PreparedMask(workspace, nhead_k, num_q_block, num_k_block, q_block_size, k_block_size, causal, cu_k, cu_nqb,

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define HBSA_ABI_VERSION 4
+#define HBSA_ABI_VERSION 5
 
 /* element types of q/k/v/out (reference: dtype follows the input tensors,
  * hbsattn/fwd_triton_auto_tile_size.py:272) */
@@ -195,6 +195,12 @@ int hbsa_fwd_static(const void *q, const void *k, const void *v, void *out,
  * of the reference kernel (reference hbsattn/fwd_triton_auto_tile_size.py:153-164: every
  * program loads one mask byte per k block of its sequence and branches on it).
  *   mask_strides  int64[3] = { mask_head, mask_qblk, mask_kblk } in elements (bytes)
+ *   total_q, total_k  token rows of the q and k/v tensors the workspace will be run with.  The sequence
+ *                 boundaries are device data the host cannot check; the pre-pass checks them against
+ *                 these bounds and the block counts, and a sequence that does not fit (q/k/v shorter than
+ *                 cu_seqlens says, inconsistent block metadata) is skipped as a whole: no kernel reads or
+ *                 writes anything for it, its output rows are left as they were.  The reference
+ *                 reads and writes out of bounds in that case.
  *
  * hbsa_fwd_run runs the attention kernel from a prepared `workspace` (same sizes, block
  * sizes and `causal` as the prepare call; q/k/v/out and softmax_scale may differ per call).
@@ -213,6 +219,7 @@ int hbsa_fwd_prepare(const int32_t *cu_q_seqlens, const int32_t *cu_k_seqlens,
                      void *workspace, size_t workspace_bytes,
                      int32_t batch, int32_t nhead_k, int32_t num_q_block, int32_t num_k_block,
                      int32_t q_block_size, int32_t k_block_size, int32_t causal,
+                     int32_t total_q, int32_t total_k,
                      const int64_t *mask_strides, void *stream);
 
 int hbsa_fwd_run(const void *q, const void *k, const void *v, void *out,

@@ -505,6 +505,38 @@ def test_clocked_walk_matches_the_oracle_and_leaves_its_clocks_at_zero(causal, k
         lib.hbsa_set_walk_min_bytes(previous)
 
 
+def test_a_sequence_that_does_not_fit_the_tensors_is_skipped_not_read_out_of_bounds():
+    """cu_seqlens that promise more tokens than q (or k, v) hold: the pre-pass checks every sequence
+    against the tensors' token counts and leaves out the one that does not fit, so the others come out
+    exactly as in the full problem and nothing beyond the tensors is touched.  (The short tensors are
+    views of the full ones, so the check is what keeps the kernels inside them, not luck.)"""
+    w = make_problem(seed=94, q_lens=[300, 500, 200], k_lens=[300, 500, 260], hq=4, hk=2, d=64, qbs=64, kbs=64, keep=0.5,
+                     diag=True, causal=True, scale=None)
+    full = _run(w)
+    args = list(w.args())
+    args[0] = w.q[:900]                       # the third sequence's queries would be rows 800 .. 999
+    out = HBSAttention(*args)
+    torch.cuda.synchronize()
+    assert out.shape[0] == 900 and torch.equal(out[:800], full[:800])
+    args = list(w.args())
+    args[1], args[2] = w.k[:1000], w.v[:1000]  # the third sequence's keys would be rows 800 .. 1059
+    out = HBSAttention(*args)
+    torch.cuda.synchronize()
+    assert torch.equal(out[:800], full[:800])
+    # and the backward: gradients of the sequences that fit are those of the full problem
+    q, k, v = (t.detach().clone().requires_grad_(True) for t in (w.q, w.k, w.v))
+    args = list(w.args())
+    args[:3] = [q, k, v]
+    dout = torch.randn_like(full)
+    HBSAttention(*args).backward(dout)
+    q2, k2, v2 = (t.detach().clone().requires_grad_(True) for t in (w.q[:900], w.k, w.v))
+    args[:3] = [q2, k2, v2]
+    HBSAttention(*args).backward(dout[:900])
+    torch.cuda.synchronize()
+    assert torch.equal(q2.grad[:800], q.grad[:800])
+    assert torch.equal(k2.grad[:800], k.grad[:800]) and torch.equal(v2.grad[:800], v.grad[:800])
+
+
 def test_prepared_masks_are_reused_only_for_unchanged_tensors():
     from hbsattn_amd import interface, set_prepared_cache_size
     w = make_problem(seed=92, q_lens=[700, 500], k_lens=[700, 900], hq=4, hk=2, d=64, qbs=64, kbs=64, keep=0.4, diag=True,
