@@ -171,7 +171,9 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out,
  * hbsa_fwd_workspace_bytes_dtype(...) exceeds HBSA_STATIC_SCRATCH_BYTES is refused with
  * HBSA_ERR_WORKSPACE_TOO_SMALL before anything is launched.  All calls on one GPU share that GPU's
  * array: calls on one stream are ordered and safe; calls that overlap on one GPU (different streams
- * or host threads) race on it and must be serialised by the caller.
+ * or host threads) race on it and must be serialised by the caller.  The first call on a device looks
+ * up the array's address and the kernels' launch limits (host-side queries, no allocation): make it
+ * before a stream capture begins, not inside one.
  */
 #define HBSA_STATIC_SCRATCH_BYTES (32u << 20)
 int hbsa_fwd_static(const void *q, const void *k, const void *v, void *out,
