@@ -24,8 +24,9 @@
 // Both recompute S.  The kept blocks of a mask row or column are found with one load per 32 or 64
 // blocks, not one per block.  A tile goes from global memory to registers while the tile before it is computed
 // on, and from registers to LDS between two barriers; a tile that is read both by rows and transposed
-// is stored twice, once in each of the forward's two swizzled layouts.  The forward's persistent
-// scheduling and LDS-DMA double buffering are not applied here yet.
+// is stored twice, once in each of the forward's two swizzled layouts.  The D = 128 dK/dV kernel instead
+// loads its tiles straight into LDS, two buffers, one layout, one barrier per tile.  The forward's
+// persistent scheduling is not applied here.
 
 namespace {
 
@@ -498,16 +499,49 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
 // operands per product) and runs eight wavefronts: wavefronts w and w + 4 own the same 32 keys and
 // take rows 0-31 and 32-63 of every tile, so that two wavefronts share a SIMD and cover each other's
 // waits; their two partial accumulators are added through LDS at the end.  No product is computed twice.
+//
+// The Q and dO tiles go from global memory straight into LDS (global_load_lds_dwordx4, 16 bytes per lane
+// to M0 + 16 * lane), two buffers each: tile t + 1 travels while tile t is computed on, one barrier per
+// tile.  A tile is read both by rows (A operand of S and dP) and transposed (A operand of the dK^T, dV^T
+// updates); one chunk swizzle serves both without bank conflicts, so it is stored once:
+// chunk ^= swz(row), swz(r) = ((r & 3) << 2) | ((r >> 2) & 3) -- a permutation of the 16 chunks over any
+// 16 consecutive rows (the reads by rows), and rows 0-7 of a group spread two each over the four
+// 64-byte column groups (the transposing reads).
+struct Dkv8Tile {
+  static constexpr int RB = 256, TILE_BYTES = 64 * RB;
+  static __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+};
+
+__device__ __forceinline__ void bwd_dma16(uint32_t lds_addr, const char *sbase, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+
+// acc[dt] += tile^T (rows 16*g .. 16*g+15 as the contraction index) . packed, tile in the Dkv8Tile layout
+template <typename E>
+__device__ __forceinline__ void dkv8_transposed_times_packed(const char *tile, int g, short8v packed, int rd_lo, int rd_hi, f32x16 *acc) {
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt) {
+    const char *a = tile + (rd_lo ^ (dt * 64)) + g * 16 * Dkv8Tile::RB;
+    const char *b = tile + (rd_hi ^ (dt * 64)) + g * 16 * Dkv8Tile::RB;
+    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(a));
+    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(b));
+    const short8v va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    acc[dt] = E::mfma(va, packed, acc[dt]);
+  }
+}
+
 template <typename E>
 __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   constexpr int D = 128;
   using T = BwdTile<D>;
+  using X = Dkv8Tile;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  char *q_rows = lds, *q_tr = lds + T::TILE_BYTES, *g_rows = lds + 2 * T::TILE_BYTES, *g_tr = lds + 3 * T::TILE_BYTES;
-  float *lse_s = (float *)(lds + 4 * T::TILE_BYTES);   // [64] log2-domain log-sum-exp of the tile's rows
-  float *dlt_s = lse_s + 64;                           // [64] their delta
-  char *k_blk = lds + 4 * T::TILE_BYTES + 512;         // [128][D] keys of the workgroup, layout read by rows
-  char *v_blk = k_blk + 2 * T::TILE_BYTES;
+  // buffer s of the tiles: Q rows at s * 2 * TILE_BYTES, dO rows one tile further (the first 64 KB, which
+  // the M0 offsets of the direct loads can address)
+  char *tiles = lds;
+  float *rowv = (float *)(lds + 4 * X::TILE_BYTES);    // buffer s: [64] log2-domain log-sum-exp of the tile's rows, [64] their delta
+  char *k_blk = lds + 4 * X::TILE_BYTES + 1024;        // [128][D] keys of the workgroup, layout read by rows
+  char *v_blk = k_blk + 2 * X::TILE_BYTES;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -604,21 +638,26 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
       qoff = -64;
     }
   };
-  // a tile's chunks over 512 threads: two per thread and tensor
-  u32x4 qt[2], gt[2];
+  // A tile's 1024 chunks over eight wavefronts: wavefront w fills rows 4 * (8 * i + w) .. + 3 with load i
+  // (i = 0, 1), lane l the 16 bytes at chunk position l % 16 of row l / 16 of those, which hold the
+  // row's chunk (l % 16) ^ swz(row).
+  const int ld_row = 4 * wave + (lane >> 4);                              // + 32 * i
+  const uint32_t ld_chunk = (uint32_t)(((lane & 15) ^ X::swz(ld_row & 15)) * 16);
+  const uint32_t q_s32 = (uint32_t)p.q_s, do_s32 = (uint32_t)p.do_s;      // the host checks that they fit
+  const uint32_t tiles_addr = (uint32_t)(uintptr_t)HBSA_AS3(tiles) + (uint32_t)wave * 1024u;
   float l2_next = INFINITY, dl_next = 0.f;
-  auto fetch = [&]() {
+  auto fetch = [&](int buf) {
     const int valid = min(64, inf.rows - qoff);
     const int64_t row_first = inf.row_begin + qoff;
     const int hq = hk * p.ratio + r;
     const char *qsrc = p.q + row_first * p.q_s + (int64_t)hq * p.q_h;
     const char *gsrc = p.dout + row_first * p.do_s + (int64_t)hq * p.do_h;
+    const uint32_t dst = tiles_addr + (uint32_t)(buf * 2 * X::TILE_BYTES);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int ch = i * 512 + threadIdx.x;
-      const int rr = min(ch / T::CPR, valid - 1), pc = ch % T::CPR;
-      qt[i] = *(const u32x4 *)(qsrc + (int64_t)rr * p.q_s + pc * 16);
-      gt[i] = *(const u32x4 *)(gsrc + (int64_t)rr * p.do_s + pc * 16);
+      const uint32_t rr = (uint32_t)min(ld_row + 32 * i, valid - 1);   // rows past the block's end repeat its last row
+      bwd_dma16(dst + (uint32_t)(i * 8 * 1024), qsrc, rr * q_s32 + ld_chunk);
+      bwd_dma16(dst + (uint32_t)(X::TILE_BYTES + i * 8 * 1024), gsrc, rr * do_s32 + ld_chunk);
     }
     l2_next = INFINITY;
     dl_next = 0.f;
@@ -628,29 +667,30 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
       dl_next = p.delta[(row_first + threadIdx.x) * p.nhead_q + hq];
     }
   };
-  const int rd = l32 * T::RB + ((g32 ^ T::swz_rows(l32)) << 4);   // this lane's 16 bytes of row l32, k-step 0
+  // this lane's operand reads: by rows (16 bytes of row l32, k-step 0) and transposed (keys 0-7 and 8-15 of a group)
+  const int rd = l32 * X::RB + ((g32 ^ X::swz(l32 & 15)) << 4);
+  const int rd_b = l32 * T::RB + ((g32 ^ T::swz_rows(l32)) << 4);   // K and V rows of the workgroup
+  const int tr_key = 4 * g32 + ((lane & 15) >> 2);
+  const int tr_lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+  const int rd_lo = tr_key * X::RB + ((tr_lc ^ X::swz(tr_key)) << 4) + 8 * (lane & 1);
+  const int rd_hi = (tr_key + 8) * X::RB + ((tr_lc ^ X::swz(tr_key + 8)) << 4) + 8 * (lane & 1);
+
   bool have = next_tile();
-  if (have) fetch();
+  int buf = 0;
+  if (have) fetch(0);
   while (have) {
     const int first_q_pos = inf.q_pos + qoff, shift = inf.shift;
-    __syncthreads();   // the previous tile has been read by every wavefront (and, the first time, K and V are in place)
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int ch = i * 512 + threadIdx.x;
-      const int rr = ch / T::CPR, pc = ch % T::CPR;
-      const int by_rows = rr * T::RB + ((pc ^ T::swz_rows(rr)) << 4), tr = rr * T::RB + ((pc ^ T::swz_tr(rr)) << 4);
-      *(u32x4 *)(q_rows + by_rows) = qt[i];
-      *(u32x4 *)(q_tr + tr) = qt[i];
-      *(u32x4 *)(g_rows + by_rows) = gt[i];
-      *(u32x4 *)(g_tr + tr) = gt[i];
-    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the tile has landed (and its lse, delta)
     if (threadIdx.x < 64) {
-      lse_s[threadIdx.x] = l2_next;
-      dlt_s[threadIdx.x] = dl_next;
+      rowv[buf * 128 + threadIdx.x] = l2_next;
+      rowv[buf * 128 + 64 + threadIdx.x] = dl_next;
     }
-    __syncthreads();
+    __syncthreads();   // ... every wavefront's; the other buffer has been read by all (and, the first time, K and V are in place)
+    const char *q_t = tiles + buf * 2 * X::TILE_BYTES, *g_t = q_t + X::TILE_BYTES;
+    const float *lse_s = rowv + buf * 128, *dlt_s = lse_s + 64;
     have = next_tile();
-    if (have) fetch();
+    if (have) fetch(buf ^ 1);
+    buf ^= 1;
     if (!active) continue;
     int first_vis = 0;
     if (p.causal) first_vis = max(0, key_pos - shift - first_q_pos);
@@ -661,9 +701,9 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
     for (int i = 0; i < 16; ++i) { sv[i] = 0.f; dp[i] = 0.f; }
 #pragma unroll
     for (int ks = 0; ks < T::KSTEPS; ++ks) {
-      const int a_off = (rd ^ (ks * 32)) + half * 32 * T::RB, b_off = (rd ^ (ks * 32)) + slot * 32 * T::RB;
-      sv = E::mfma(*(const short8v *)(q_rows + a_off), *(const short8v *)(k_blk + b_off), sv);
-      dp = E::mfma(*(const short8v *)(g_rows + a_off), *(const short8v *)(v_blk + b_off), dp);
+      const int a_off = (rd ^ (ks * 32)) + half * 32 * X::RB, b_off = (rd_b ^ (ks * 32)) + slot * 32 * T::RB;
+      sv = E::mfma(*(const short8v *)(q_t + a_off), *(const short8v *)(k_blk + b_off), sv);
+      dp = E::mfma(*(const short8v *)(g_t + a_off), *(const short8v *)(v_blk + b_off), dp);
     }
     float ep[16], ed[16];
 #pragma unroll
@@ -682,10 +722,10 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
     short8v plo, phi, dlo, dhi;
     bwd_pack<E>(ep, plo, phi);
     bwd_pack<E>(ed, dlo, dhi);
-    bwd_transposed_times_packed<D, E>(g_tr, 2 * half, plo, lane, acc_v);
-    bwd_transposed_times_packed<D, E>(g_tr, 2 * half + 1, phi, lane, acc_v);
-    bwd_transposed_times_packed<D, E>(q_tr, 2 * half, dlo, lane, acc_k);
-    bwd_transposed_times_packed<D, E>(q_tr, 2 * half + 1, dhi, lane, acc_k);
+    dkv8_transposed_times_packed<E>(g_t, 2 * half, plo, rd_lo, rd_hi, acc_v);
+    dkv8_transposed_times_packed<E>(g_t, 2 * half + 1, phi, rd_lo, rd_hi, acc_v);
+    dkv8_transposed_times_packed<E>(q_t, 2 * half, dlo, rd_lo, rd_hi, acc_k);
+    dkv8_transposed_times_packed<E>(q_t, 2 * half + 1, dhi, rd_lo, rd_hi, acc_k);
   }
   // wavefronts 4-7 hand their partial sums to wavefronts 0-3 through LDS: [slot][register][lane] floats
   __syncthreads();
@@ -722,7 +762,7 @@ int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_
   const int64_t rows = (int64_t)dp.total_q * dp.nhead_q;
   hipLaunchKernelGGL((hbsa_bwd_delta_kernel<D, E>), dim3((unsigned)((rows * (D / 8) + 255) / 256)), dim3(256), 0, stream, dp);
   // D = 128: tiles, the rows' lse and delta, K and V of the workgroup; at least the 128 KB of the final exchange
-  const int lds_dq = 3 * T::TILE_BYTES, lds_dkv = D == 128 ? 8 * T::TILE_BYTES + 512 : 4 * T::TILE_BYTES + 512;
+  const int lds_dq = 3 * T::TILE_BYTES, lds_dkv = D == 128 ? 8 * T::TILE_BYTES + 1024 : 4 * T::TILE_BYTES + 512;
   if (lds_dkv > 48 * 1024) {
     static thread_local bool raised[kMaxDevices] = {};
     int dev = 0;
