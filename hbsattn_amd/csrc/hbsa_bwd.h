@@ -88,7 +88,23 @@ struct BwdTile {
   // chunk swizzles of the forward's K tile (read by rows) and V tile (read transposed)
   static __device__ __forceinline__ int swz_rows(int r) { return (r / RPG) % CPR; }
   static __device__ __forceinline__ int swz_tr(int r) { return CPR >= 8 ? (((r / RPG) % (CPR / 4)) << 2) : 0; }
+  // One chunk swizzle for a tile that is read both ways, so that it is stored once (the tiles that go from
+  // global memory straight into LDS): with a = (r / RPG) % CPR, the bits of a rotated so that its lowest
+  // bits select the 64-byte column group.  Over any 16 consecutive rows the 16-byte slots of a chunk
+  // column are all different (reads by rows), and rows 0-7 of a group spread evenly over the column
+  // groups (transposing reads).
+  static __device__ __forceinline__ int swz_both(int r) {
+    const int a = (r / RPG) % CPR;
+    if constexpr (CPR == 16) return ((a & 3) << 2) | (a >> 2);
+    else if constexpr (CPR == 8) return ((a & 1) << 2) | (a >> 1);
+    else return a;
+  }
 };
+
+// 16 bytes per lane from global memory (scalar base + 32-bit lane offset) straight into LDS at lds_addr + 16 * lane
+__device__ __forceinline__ void bwd_dma16(uint32_t lds_addr, const char *sbase, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+}
 
 // A 64-row tile on its way from global memory to LDS: each thread holds LOADS 16-byte chunks.  The
 // fetch of the next tile is issued before the current one is computed on, so its latency hides
@@ -123,11 +139,11 @@ __device__ __forceinline__ void bwd_stash_tile(const BwdTileRegs<D> &t, char *by
 }
 
 // rows 32*h .. 32*h+31 of the tile . frag^T, the forward's S^T = K Q^T for one half of a tile
-template <int D, typename E>
+template <int D, typename E, bool BOTH = false>
 __device__ __forceinline__ f32x16 bwd_rows_times_frag(const char *tile, int h, const short8v *frag, int lane) {
   using T = BwdTile<D>;
   const int l32 = lane & 31, g32 = lane >> 5;
-  const int rd = l32 * T::RB + ((g32 ^ T::swz_rows(l32)) << 4) + h * 32 * T::RB;
+  const int rd = l32 * T::RB + ((g32 ^ (BOTH ? T::swz_both(l32) : T::swz_rows(l32))) << 4) + h * 32 * T::RB;
   f32x16 a;
 #pragma unroll
   for (int i = 0; i < 16; ++i) a[i] = 0.f;
@@ -138,19 +154,21 @@ __device__ __forceinline__ f32x16 bwd_rows_times_frag(const char *tile, int h, c
 
 // acc[dt] += tile^T (rows 16*g .. 16*g+15 of the tile as the contraction index) . packed, the forward's
 // O^T += V^T P^T for one group of 16 keys
-template <int D, typename E>
+template <int D, typename E, bool BOTH = false>
 __device__ __forceinline__ void bwd_transposed_times_packed(const char *tile, int g, short8v packed, int lane, f32x16 *acc) {
   using T = BwdTile<D>;
   const int g32 = lane >> 5;
   const int key = 4 * g32 + ((lane & 15) >> 2);
   const int lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-  const int rd = key * T::RB + ((lc | T::swz_tr(key)) << 4) + 8 * (lane & 1);
+  const int rd = key * T::RB + ((BOTH ? lc ^ T::swz_both(key) : lc | T::swz_tr(key)) << 4) + 8 * (lane & 1);
+  // (keys 8 further down: the same chunk position in the forward's layout, its own in the other)
+  const int rd8 = BOTH ? (key + 8) * T::RB + ((lc ^ T::swz_both(key + 8)) << 4) + 8 * (lane & 1) : rd + 8 * T::RB;
 #pragma unroll
   for (int dt = 0; dt < T::DT; ++dt) {
     const char *a = tile + (rd ^ (dt * 64)) + g * 16 * T::RB;
+    const char *a8 = tile + (rd8 ^ (dt * 64)) + g * 16 * T::RB;
     const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(a));
-    const short4v hi =
-        __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(a + 8 * T::RB));
+    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(a8));
     const short8v va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     acc[dt] = E::mfma(va, packed, acc[dt]);
   }
@@ -187,7 +205,8 @@ template <int D, typename E>
 __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   using T = BwdTile<D>;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  char *k_rows = lds, *k_tr = lds + T::TILE_BYTES, *v_rows = lds + 2 * T::TILE_BYTES;
+  // two buffers of a K tile followed by a V tile, filled straight from global memory, in the layout
+  // that serves the reads by rows and the transposing reads (BwdTile::swz_both)
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -261,31 +280,44 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
     return true;
   };
   auto tile_valid = [&]() { return min(kTileKeys, min((j + 1) * p.kbs, inf.kmax) - kpos); };
-  BwdTileRegs<D> kt, vt;
+  // A tile's chunks over four wavefronts: one load of a wavefront fills 1024 bytes (RPL rows); load i of
+  // wavefront w the rows RPL * (4 * i + w) .. + RPL - 1; lane l the chunk position l % CPR of row l / CPR
+  // of those, which holds the row's chunk (l % CPR) ^ swz_both(row).
+  constexpr int RPL = 1024 / T::RB, LOADS = 64 / (4 * RPL);
+  const int ld_row = RPL * wave + lane / T::CPR;                                  // + 4 * RPL * i
+  const uint32_t ld_chunk = (uint32_t)(((lane % T::CPR) ^ T::swz_both(ld_row)) * 16);
+  const uint32_t k_s32 = (uint32_t)p.k_s, v_s32 = (uint32_t)p.v_s;              // the host checks that they fit
+  const uint32_t tiles_addr = (uint32_t)(uintptr_t)HBSA_AS3(lds) + (uint32_t)wave * 1024u;
+  auto fetch = [&](int buf) {   // the tile next_tile() has just moved to
+    const int valid = tile_valid();
+    const char *ksrc = kg + (int64_t)kpos * p.k_s, *vsrc = vg + (int64_t)kpos * p.v_s;
+    const uint32_t dst = tiles_addr + (uint32_t)(buf * 2 * T::TILE_BYTES);
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const uint32_t rr = (uint32_t)min(ld_row + 4 * RPL * i, valid - 1);   // rows past the end repeat the last one (masked later)
+      bwd_dma16(dst + (uint32_t)(i * 4 * 1024), ksrc, rr * k_s32 + ld_chunk);
+      bwd_dma16(dst + (uint32_t)(T::TILE_BYTES + i * 4 * 1024), vsrc, rr * v_s32 + ld_chunk);
+    }
+  };
   bool have = next_tile();
-  if (have) {
-    bwd_fetch_tile<D>(kg + (int64_t)kpos * p.k_s, p.k_s, tile_valid(), kt);
-    bwd_fetch_tile<D>(vg + (int64_t)kpos * p.v_s, p.v_s, tile_valid(), vt);
-  }
+  int buf = 0;
+  if (have) fetch(0);
   while (have) {
     const int cur_kpos = kpos, valid = tile_valid();
-    __syncthreads();   // the previous tile has been read by every wavefront
-    bwd_stash_tile<D>(kt, k_rows, k_tr);
-    bwd_stash_tile<D>(vt, v_rows, nullptr);
-    __syncthreads();
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the tile has landed
+    __syncthreads();                      // ... every wavefront's, and the other buffer has been read by all
+    const char *k_t = lds + buf * 2 * T::TILE_BYTES, *v_t = k_t + T::TILE_BYTES;
     have = next_tile();
-    if (have) {   // on its way while this tile is computed on
-      bwd_fetch_tile<D>(kg + (int64_t)kpos * p.k_s, p.k_s, tile_valid(), kt);
-      bwd_fetch_tile<D>(vg + (int64_t)kpos * p.v_s, p.v_s, tile_valid(), vt);
-    }
+    if (have) fetch(buf ^ 1);   // on its way while this tile is computed on
+    buf ^= 1;
     if (!active) continue;
     int lim = valid;   // keys of the tile below lim are visible to this lane's row
     if (p.causal) lim = min(lim, lane_kvis - cur_kpos + 1);
     lim -= 4 * g32;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const f32x16 s = bwd_rows_times_frag<D, E>(k_rows, h, qf, lane);
-      const f32x16 dp = bwd_rows_times_frag<D, E>(v_rows, h, dof, lane);
+      const f32x16 s = bwd_rows_times_frag<D, E, true>(k_t, h, qf, lane);
+      const f32x16 dp = bwd_rows_times_frag<D, E, true>(v_t, h, dof, lane);
       float e[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -295,8 +327,8 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
       }
       short8v lo, hi;
       bwd_pack<E>(e, lo, hi);
-      bwd_transposed_times_packed<D, E>(k_tr, 2 * h, lo, lane, acc);
-      bwd_transposed_times_packed<D, E>(k_tr, 2 * h + 1, hi, lane, acc);
+      bwd_transposed_times_packed<D, E, true>(k_t, 2 * h, lo, lane, acc);
+      bwd_transposed_times_packed<D, E, true>(k_t, 2 * h + 1, hi, lane, acc);
     }
   }
   if (active && l32 < nrows)
@@ -511,10 +543,6 @@ struct Dkv8Tile {
   static constexpr int RB = 256, TILE_BYTES = 64 * RB;
   static __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
 };
-
-__device__ __forceinline__ void bwd_dma16(uint32_t lds_addr, const char *sbase, uint32_t voff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
-}
 
 // acc[dt] += tile^T (rows 16*g .. 16*g+15 as the contraction index) . packed, tile in the Dkv8Tile layout
 template <typename E>
@@ -762,7 +790,7 @@ int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_
   const int64_t rows = (int64_t)dp.total_q * dp.nhead_q;
   hipLaunchKernelGGL((hbsa_bwd_delta_kernel<D, E>), dim3((unsigned)((rows * (D / 8) + 255) / 256)), dim3(256), 0, stream, dp);
   // D = 128: tiles, the rows' lse and delta, K and V of the workgroup; at least the 128 KB of the final exchange
-  const int lds_dq = 3 * T::TILE_BYTES, lds_dkv = D == 128 ? 8 * T::TILE_BYTES + 1024 : 4 * T::TILE_BYTES + 512;
+  const int lds_dq = 4 * T::TILE_BYTES, lds_dkv = D == 128 ? 8 * T::TILE_BYTES + 1024 : 4 * T::TILE_BYTES + 512;
   if (lds_dkv > 48 * 1024) {
     static thread_local bool raised[kMaxDevices] = {};
     int dev = 0;
