@@ -95,7 +95,10 @@ def test_empty_problem_is_a_no_op():
 
 
 def _call_bwd(lib, **over):
-    strides = (ctypes.c_int64 * 16)(*([4096, 128] * 8))
+    values = [4096, 128] * 8
+    for i, v in over.pop("strides", {}).items():
+        values[i] = v
+    strides = (ctypes.c_int64 * 16)(*values)
     a = dict(q=256, k=256, v=256, out=256, dout=256, lse=256, dq=256, dk=256, dv=256, cu_k=256, cu_nqb=256, cu_nkb=256,
              ws=256, ws_bytes=1 << 30, bws=256, bws_bytes=1 << 30, dtype=0, batch=1, total_q=128, total_k=128, hq=32, hk=32,
              d=128, nqb=1, nkb=1, qbs=128, kbs=128, causal=1, scale=0.1)
@@ -114,6 +117,9 @@ def _call_bwd(lib, **over):
     (dict(dq=264), -1, "aligned"),
     (dict(ws_bytes=16), -3, "workspace"),
     (dict(bws_bytes=16), -3, "bwd_workspace"),
+    (dict(strides={2: -4096}), -2, "k/v token stride"),          # tile rows are addressed with 32-bit offsets
+    (dict(strides={4: 1 << 25}), -2, "k/v token stride"),
+    (dict(strides={8: -4096}), -2, "q/dout token stride"),
 ])
 def test_backward_argument_validation_without_touching_the_gpu(over, code, needle):
     lib = _lib.load()
