@@ -535,22 +535,15 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
 // The Q and dO tiles go from global memory straight into LDS (global_load_lds_dwordx4, 16 bytes per lane
 // to M0 + 16 * lane), two buffers each: tile t + 1 travels while tile t is computed on, one barrier per
 // tile.  A tile is read both by rows (A operand of S and dP) and transposed (A operand of the dK^T, dV^T
-// updates); one chunk swizzle serves both without bank conflicts, so it is stored once:
-// chunk ^= swz(row), swz(r) = ((r & 3) << 2) | ((r >> 2) & 3) -- a permutation of the 16 chunks over any
-// 16 consecutive rows (the reads by rows), and rows 0-7 of a group spread two each over the four
-// 64-byte column groups (the transposing reads).
-struct Dkv8Tile {
-  static constexpr int RB = 256, TILE_BYTES = 64 * RB;
-  static __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
-};
+// updates) and is stored once, in the layout of BwdTile::swz_both.
 
-// acc[dt] += tile^T (rows 16*g .. 16*g+15 as the contraction index) . packed, tile in the Dkv8Tile layout
+// acc[dt] += tile^T (rows 16*g .. 16*g+15 as the contraction index) . packed, tile in the swz_both layout
 template <typename E>
 __device__ __forceinline__ void dkv8_transposed_times_packed(const char *tile, int g, short8v packed, int rd_lo, int rd_hi, f32x16 *acc) {
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt) {
-    const char *a = tile + (rd_lo ^ (dt * 64)) + g * 16 * Dkv8Tile::RB;
-    const char *b = tile + (rd_hi ^ (dt * 64)) + g * 16 * Dkv8Tile::RB;
+    const char *a = tile + (rd_lo ^ (dt * 64)) + g * 16 * BwdTile<128>::RB;
+    const char *b = tile + (rd_hi ^ (dt * 64)) + g * 16 * BwdTile<128>::RB;
     const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(a));
     const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(b));
     const short8v va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -562,14 +555,13 @@ template <typename E>
 __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   constexpr int D = 128;
   using T = BwdTile<D>;
-  using X = Dkv8Tile;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   // buffer s of the tiles: Q rows at s * 2 * TILE_BYTES, dO rows one tile further (the first 64 KB, which
   // the M0 offsets of the direct loads can address)
   char *tiles = lds;
-  float *rowv = (float *)(lds + 4 * X::TILE_BYTES);    // buffer s: [64] log2-domain log-sum-exp of the tile's rows, [64] their delta
-  char *k_blk = lds + 4 * X::TILE_BYTES + 1024;        // [128][D] keys of the workgroup, layout read by rows
-  char *v_blk = k_blk + 2 * X::TILE_BYTES;
+  float *rowv = (float *)(lds + 4 * T::TILE_BYTES);    // buffer s: [64] log2-domain log-sum-exp of the tile's rows, [64] their delta
+  char *k_blk = lds + 4 * T::TILE_BYTES + 1024;        // [128][D] keys of the workgroup, layout read by rows
+  char *v_blk = k_blk + 2 * T::TILE_BYTES;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -670,7 +662,7 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   // (i = 0, 1), lane l the 16 bytes at chunk position l % 16 of row l / 16 of those, which hold the
   // row's chunk (l % 16) ^ swz(row).
   const int ld_row = 4 * wave + (lane >> 4);                              // + 32 * i
-  const uint32_t ld_chunk = (uint32_t)(((lane & 15) ^ X::swz(ld_row & 15)) * 16);
+  const uint32_t ld_chunk = (uint32_t)(((lane & 15) ^ T::swz_both(ld_row & 15)) * 16);
   const uint32_t q_s32 = (uint32_t)p.q_s, do_s32 = (uint32_t)p.do_s;      // the host checks that they fit
   const uint32_t tiles_addr = (uint32_t)(uintptr_t)HBSA_AS3(tiles) + (uint32_t)wave * 1024u;
   float l2_next = INFINITY, dl_next = 0.f;
@@ -680,12 +672,12 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
     const int hq = hk * p.ratio + r;
     const char *qsrc = p.q + row_first * p.q_s + (int64_t)hq * p.q_h;
     const char *gsrc = p.dout + row_first * p.do_s + (int64_t)hq * p.do_h;
-    const uint32_t dst = tiles_addr + (uint32_t)(buf * 2 * X::TILE_BYTES);
+    const uint32_t dst = tiles_addr + (uint32_t)(buf * 2 * T::TILE_BYTES);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const uint32_t rr = (uint32_t)min(ld_row + 32 * i, valid - 1);   // rows past the block's end repeat its last row
       bwd_dma16(dst + (uint32_t)(i * 8 * 1024), qsrc, rr * q_s32 + ld_chunk);
-      bwd_dma16(dst + (uint32_t)(X::TILE_BYTES + i * 8 * 1024), gsrc, rr * do_s32 + ld_chunk);
+      bwd_dma16(dst + (uint32_t)(T::TILE_BYTES + i * 8 * 1024), gsrc, rr * do_s32 + ld_chunk);
     }
     l2_next = INFINITY;
     dl_next = 0.f;
@@ -696,12 +688,12 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
     }
   };
   // this lane's operand reads: by rows (16 bytes of row l32, k-step 0) and transposed (keys 0-7 and 8-15 of a group)
-  const int rd = l32 * X::RB + ((g32 ^ X::swz(l32 & 15)) << 4);
+  const int rd = l32 * T::RB + ((g32 ^ T::swz_both(l32 & 15)) << 4);
   const int rd_b = l32 * T::RB + ((g32 ^ T::swz_rows(l32)) << 4);   // K and V rows of the workgroup
   const int tr_key = 4 * g32 + ((lane & 15) >> 2);
   const int tr_lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-  const int rd_lo = tr_key * X::RB + ((tr_lc ^ X::swz(tr_key)) << 4) + 8 * (lane & 1);
-  const int rd_hi = (tr_key + 8) * X::RB + ((tr_lc ^ X::swz(tr_key + 8)) << 4) + 8 * (lane & 1);
+  const int rd_lo = tr_key * T::RB + ((tr_lc ^ T::swz_both(tr_key)) << 4) + 8 * (lane & 1);
+  const int rd_hi = (tr_key + 8) * T::RB + ((tr_lc ^ T::swz_both(tr_key + 8)) << 4) + 8 * (lane & 1);
 
   bool have = next_tile();
   int buf = 0;
@@ -714,7 +706,7 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
       rowv[buf * 128 + 64 + threadIdx.x] = dl_next;
     }
     __syncthreads();   // ... every wavefront's; the other buffer has been read by all (and, the first time, K and V are in place)
-    const char *q_t = tiles + buf * 2 * X::TILE_BYTES, *g_t = q_t + X::TILE_BYTES;
+    const char *q_t = tiles + buf * 2 * T::TILE_BYTES, *g_t = q_t + T::TILE_BYTES;
     const float *lse_s = rowv + buf * 128, *dlt_s = lse_s + 64;
     have = next_tile();
     if (have) fetch(buf ^ 1);
@@ -729,7 +721,7 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
     for (int i = 0; i < 16; ++i) { sv[i] = 0.f; dp[i] = 0.f; }
 #pragma unroll
     for (int ks = 0; ks < T::KSTEPS; ++ks) {
-      const int a_off = (rd ^ (ks * 32)) + half * 32 * X::RB, b_off = (rd_b ^ (ks * 32)) + slot * 32 * T::RB;
+      const int a_off = (rd ^ (ks * 32)) + half * 32 * T::RB, b_off = (rd_b ^ (ks * 32)) + slot * 32 * T::RB;
       sv = E::mfma(*(const short8v *)(q_t + a_off), *(const short8v *)(k_blk + b_off), sv);
       dp = E::mfma(*(const short8v *)(g_t + a_off), *(const short8v *)(v_blk + b_off), dp);
     }
