@@ -135,6 +135,37 @@ def test_gqa_gradients_equal_mha_with_repeated_kv_heads():
     torch.testing.assert_close(dv.float(), dv4.float().sum(dim=1, keepdim=True), atol=3e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("d", [32, 64, 128])
+def test_strided_tensors_give_the_gradients_of_their_contiguous_copies(d):
+    # q, k, v as slices of one packed [tokens, 3, heads, d] tensor (token stride 3 * heads * d), dout and out stored
+    # head-major ([heads, tokens, d] seen through a transpose: token stride d): the kernels address tile rows by
+    # 32-bit offsets built from these strides
+    from hbsattn_amd import interface as I
+    from hbsattn_amd import calculate_blocks
+    heads, qbs, kbs = 2, 64, 128
+    q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(40 + d, [300, 130], [300, 130], heads, heads, d, qbs, kbs, 0.6, torch.bfloat16)
+    print(f"backward strided d={d}", flush=True)
+    packed = torch.stack([q, k, v], dim=1).cuda()                       # [tokens, 3, heads, d]
+    qs, ks, vs = packed[:, 0], packed[:, 1], packed[:, 2]
+    assert not qs.is_contiguous() and qs.stride(0) == 3 * heads * d
+    nq, _, qb2b, cu_nqb = calculate_blocks(cq, qbs)
+    nk, _, _, cu_nkb = calculate_blocks(ck, kbs)
+    prepared = I.hbsa_prepare(cq, ck, mask.cuda(), qbs, kbs, True, int(nq), qb2b, cu_nqb, int(nk), cu_nkb)
+    out, lse = I.hbsa_run(qs, ks, vs, prepared, None, return_lse=True)
+    out_hm = out.transpose(0, 1).contiguous().transpose(0, 1)           # same values, [heads, tokens, d] in memory
+    do_hm = do.cuda().transpose(0, 1).contiguous().transpose(0, 1)
+    assert do_hm.stride(0) == d and not do_hm.is_contiguous()
+    got = I.hbsa_backward(qs, ks, vs, out_hm, do_hm, lse, prepared, None)
+    want = I.hbsa_backward(qs.contiguous(), ks.contiguous(), vs.contiguous(), out.contiguous(), do.cuda(), lse, prepared, None)
+    torch.cuda.synchronize()
+    for g, w in zip(got, want):
+        assert torch.equal(g, w)
+    rdq, rdk, rdv = hbsa_oracle_grads(q, k, v, do, cu_q, cu_k, mask, qbs, kbs, True, None)
+    _check(got[0], rdq, "dq")
+    _check(got[1], rdk, "dk")
+    _check(got[2], rdv, "dv")
+
+
 def test_float32_inputs_still_raise_like_the_reference():
     from hbsattn_amd import HBSAttention
     q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(14, [64], [64], 2, 2, 32, 32, 32, 1.1, torch.float32)
