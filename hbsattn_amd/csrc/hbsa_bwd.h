@@ -22,11 +22,10 @@
 //                           every q head of the group) stream through LDS in 64-row tiles:
 //                           S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS.
 // Both recompute S.  The kept blocks of a mask row or column are found with one load per 32 or 64
-// blocks, not one per block.  A tile goes from global memory to registers while the tile before it is computed
-// on, and from registers to LDS between two barriers; a tile that is read both by rows and transposed
-// is stored twice, once in each of the forward's two swizzled layouts.  The D = 128 dK/dV kernel instead
-// loads its tiles straight into LDS, two buffers, one layout, one barrier per tile.  The forward's
-// persistent scheduling is not applied here.
+// blocks, not one per block.  Tiles go from global memory straight into LDS (global_load_lds_dwordx4),
+// two buffers: tile t + 1 travels while tile t is computed on, one barrier per tile.  A tile that is
+// read both by rows and transposed is stored once, in a layout without bank conflicts for either
+// (BwdTile::swz_both).  The forward's persistent scheduling is not applied here.
 
 namespace {
 
@@ -87,7 +86,6 @@ struct BwdTile {
   static constexpr int DT = D / 32;
   // chunk swizzles of the forward's K tile (read by rows) and V tile (read transposed)
   static __device__ __forceinline__ int swz_rows(int r) { return (r / RPG) % CPR; }
-  static __device__ __forceinline__ int swz_tr(int r) { return CPR >= 8 ? (((r / RPG) % (CPR / 4)) << 2) : 0; }
   // One chunk swizzle for a tile that is read both ways, so that it is stored once (the tiles that go from
   // global memory straight into LDS): with a = (r / RPG) % CPR, the bits of a rotated so that its lowest
   // bits select the 64-byte column group.  Over any 16 consecutive rows the 16-byte slots of a chunk
@@ -106,44 +104,12 @@ __device__ __forceinline__ void bwd_dma16(uint32_t lds_addr, const char *sbase, 
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
 }
 
-// A 64-row tile on its way from global memory to LDS: each thread holds LOADS 16-byte chunks.  The
-// fetch of the next tile is issued before the current one is computed on, so its latency hides
-// behind the matrix work; bwd_stash_tile writes the chunks to LDS once the buffers are free again.
-template <int D>
-struct BwdTileRegs {
-  static constexpr int LOADS = 64 * BwdTile<D>::CPR / 256;
-  u32x4 x[LOADS];
-};
-// 64 rows of `src` (row stride `stride` bytes; rows past `valid` repeat the last valid one)
-template <int D>
-__device__ __forceinline__ void bwd_fetch_tile(const char *src, int64_t stride, int valid, BwdTileRegs<D> &t) {
-  using T = BwdTile<D>;
-#pragma unroll
-  for (int i = 0; i < BwdTileRegs<D>::LOADS; ++i) {
-    const int ch = i * 256 + threadIdx.x;
-    const int r = ch / T::CPR, pc = ch % T::CPR;
-    t.x[i] = *(const u32x4 *)(src + (int64_t)min(r, valid - 1) * stride + pc * 16);
-  }
-}
-// `by_rows`: the layout read by rows; `transposed` (may be null): the layout read transposed
-template <int D>
-__device__ __forceinline__ void bwd_stash_tile(const BwdTileRegs<D> &t, char *by_rows, char *transposed) {
-  using T = BwdTile<D>;
-#pragma unroll
-  for (int i = 0; i < BwdTileRegs<D>::LOADS; ++i) {
-    const int ch = i * 256 + threadIdx.x;
-    const int r = ch / T::CPR, pc = ch % T::CPR;
-    *(u32x4 *)(by_rows + r * T::RB + ((pc ^ T::swz_rows(r)) << 4)) = t.x[i];
-    if (transposed != nullptr) *(u32x4 *)(transposed + r * T::RB + ((pc ^ T::swz_tr(r)) << 4)) = t.x[i];
-  }
-}
-
 // rows 32*h .. 32*h+31 of the tile . frag^T, the forward's S^T = K Q^T for one half of a tile
-template <int D, typename E, bool BOTH = false>
+template <int D, typename E>
 __device__ __forceinline__ f32x16 bwd_rows_times_frag(const char *tile, int h, const short8v *frag, int lane) {
   using T = BwdTile<D>;
   const int l32 = lane & 31, g32 = lane >> 5;
-  const int rd = l32 * T::RB + ((g32 ^ (BOTH ? T::swz_both(l32) : T::swz_rows(l32))) << 4) + h * 32 * T::RB;
+  const int rd = l32 * T::RB + ((g32 ^ T::swz_both(l32)) << 4) + h * 32 * T::RB;
   f32x16 a;
 #pragma unroll
   for (int i = 0; i < 16; ++i) a[i] = 0.f;
@@ -154,15 +120,14 @@ __device__ __forceinline__ f32x16 bwd_rows_times_frag(const char *tile, int h, c
 
 // acc[dt] += tile^T (rows 16*g .. 16*g+15 of the tile as the contraction index) . packed, the forward's
 // O^T += V^T P^T for one group of 16 keys
-template <int D, typename E, bool BOTH = false>
+template <int D, typename E>
 __device__ __forceinline__ void bwd_transposed_times_packed(const char *tile, int g, short8v packed, int lane, f32x16 *acc) {
   using T = BwdTile<D>;
   const int g32 = lane >> 5;
   const int key = 4 * g32 + ((lane & 15) >> 2);
   const int lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-  const int rd = key * T::RB + ((BOTH ? lc ^ T::swz_both(key) : lc | T::swz_tr(key)) << 4) + 8 * (lane & 1);
-  // (keys 8 further down: the same chunk position in the forward's layout, its own in the other)
-  const int rd8 = BOTH ? (key + 8) * T::RB + ((lc ^ T::swz_both(key + 8)) << 4) + 8 * (lane & 1) : rd + 8 * T::RB;
+  const int rd = key * T::RB + ((lc ^ T::swz_both(key)) << 4) + 8 * (lane & 1);
+  const int rd8 = (key + 8) * T::RB + ((lc ^ T::swz_both(key + 8)) << 4) + 8 * (lane & 1);   // the row 8 further down
 #pragma unroll
   for (int dt = 0; dt < T::DT; ++dt) {
     const char *a = tile + (rd ^ (dt * 64)) + g * 16 * T::RB;
@@ -316,8 +281,8 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
     lim -= 4 * g32;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const f32x16 s = bwd_rows_times_frag<D, E, true>(k_t, h, qf, lane);
-      const f32x16 dp = bwd_rows_times_frag<D, E, true>(v_t, h, dof, lane);
+      const f32x16 s = bwd_rows_times_frag<D, E>(k_t, h, qf, lane);
+      const f32x16 dp = bwd_rows_times_frag<D, E>(v_t, h, dof, lane);
       float e[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -327,22 +292,27 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
       }
       short8v lo, hi;
       bwd_pack<E>(e, lo, hi);
-      bwd_transposed_times_packed<D, E, true>(k_t, 2 * h, lo, lane, acc);
-      bwd_transposed_times_packed<D, E, true>(k_t, 2 * h + 1, hi, lane, acc);
+      bwd_transposed_times_packed<D, E>(k_t, 2 * h, lo, lane, acc);
+      bwd_transposed_times_packed<D, E>(k_t, 2 * h + 1, hi, lane, acc);
     }
   }
   if (active && l32 < nrows)
     bwd_store_rows<D, E>(p.dq + (int64_t)(inf.row_begin + row0 + l32) * p.dq_s + (int64_t)hq * p.dq_h, acc, p.scale, g32);
 }
 
-// ---- dK, dV ------------------------------------------------------------------------------------------
+// ---- dK, dV (head dims up to 64) ---------------------------------------------------------------------
+// Four wavefronts; K^T and V^T of a wavefront's 32 keys stay in registers.  The Q and dO tiles go straight
+// into LDS like the dQ kernel's (two buffers, one layout, one barrier per tile).  When the workgroup's keys
+// fill at most two 32-key slots (k blocks of up to 64 keys, or the narrow rest of a wider block), two
+// wavefronts share a slot and take the upper and lower 32 rows of every tile; their partial sums are added
+// through LDS at the end, as in the D = 128 kernel below.
 template <int D, typename E>
-__global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel(BwdParams p) {
+__global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dkv_kernel(BwdParams p) {
+  static_assert(D <= 64, "head dim 128 has its own kernel");
   using T = BwdTile<D>;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  char *q_rows = lds, *q_tr = lds + T::TILE_BYTES, *g_rows = lds + 2 * T::TILE_BYTES, *g_tr = lds + 3 * T::TILE_BYTES;
-  float *lse_s = (float *)(lds + 4 * T::TILE_BYTES);   // [64] log2-domain log-sum-exp of the tile's rows
-  float *dlt_s = lse_s + 64;                           // [64] their delta
+  // buffer s of the tiles: Q rows at s * 2 * TILE_BYTES, dO rows one tile further
+  float *rowv = (float *)(lds + 4 * T::TILE_BYTES);    // buffer s: [64] log2-domain log-sum-exp of the tile's rows, [64] their delta
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -368,7 +338,11 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
   const int kbl = kb - p.cu_num_k_block[b];          // in-sequence index of the k block
   const int k0 = p.cu_k[b], klen = p.cu_k[b + 1] - k0;
   const int krows = min(p.kbs, klen - kbl * p.kbs);  // keys in the block
-  const int row0 = (sub * 4 + wave) * kWaveRows;
+  const int wg_keys = min(4 * kWaveRows, p.kbs - sub * 4 * kWaveRows);   // by the block size: the same for every k block
+  const bool shared_slots = wg_keys <= 2 * kWaveRows;                    // two wavefronts per 32-key slot
+  const int slot = shared_slots ? (wave & 1) : wave;
+  const int part = shared_slots ? (wave >> 1) : 0;                       // which 32 rows of a tile (shared slots)
+  const int row0 = (sub * 4 + slot) * kWaveRows;
   const int nrows = min(kWaveRows, krows - row0);
   const bool active = nrows > 0;
   const int key_pos = kbl * p.kbs + min(row0 + l32, krows - 1);   // in-sequence position of this lane's key
@@ -439,14 +413,26 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
       qoff = -64;   // the step above moves to the block's first tile
     }
   };
-  BwdTileRegs<D> qt, gt;
+  // (placement of a tile's chunks over the four wavefronts: see hbsa_bwd_dq_kernel)
+  constexpr int RPL = 1024 / T::RB, LOADS = 64 / (4 * RPL);
+  const int ld_row = RPL * wave + lane / T::CPR;
+  const uint32_t ld_chunk = (uint32_t)(((lane % T::CPR) ^ T::swz_both(ld_row)) * 16);
+  const uint32_t q_s32 = (uint32_t)p.q_s, do_s32 = (uint32_t)p.do_s;   // the host checks that they fit
+  const uint32_t tiles_addr = (uint32_t)(uintptr_t)HBSA_AS3(lds) + (uint32_t)wave * 1024u;
   float l2_next = INFINITY, dl_next = 0.f;   // threads 0-63: log2-domain log-sum-exp and delta of the tile's row
-  auto fetch = [&]() {
+  auto fetch = [&](int buf) {
     const int valid = min(64, inf.rows - qoff);
     const int64_t row_first = inf.row_begin + qoff;
     const int hq = hk * p.ratio + r;
-    bwd_fetch_tile<D>(p.q + row_first * p.q_s + (int64_t)hq * p.q_h, p.q_s, valid, qt);
-    bwd_fetch_tile<D>(p.dout + row_first * p.do_s + (int64_t)hq * p.do_h, p.do_s, valid, gt);
+    const char *qsrc = p.q + row_first * p.q_s + (int64_t)hq * p.q_h;
+    const char *gsrc = p.dout + row_first * p.do_s + (int64_t)hq * p.do_h;
+    const uint32_t dst = tiles_addr + (uint32_t)(buf * 2 * T::TILE_BYTES);
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const uint32_t rr = (uint32_t)min(ld_row + 4 * RPL * i, valid - 1);   // rows past the block's end repeat its last row
+      bwd_dma16(dst + (uint32_t)(i * 4 * 1024), qsrc, rr * q_s32 + ld_chunk);
+      bwd_dma16(dst + (uint32_t)(T::TILE_BYTES + i * 4 * 1024), gsrc, rr * do_s32 + ld_chunk);
+    }
     l2_next = INFINITY;   // rows past the block's end take no part: P = exp2(-inf) = 0
     dl_next = 0.f;
     if (threadIdx.x < valid) {
@@ -456,45 +442,31 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
     }
   };
   bool have = next_tile();
-  if (have) fetch();
+  int buf = 0;
+  if (have) fetch(0);
   while (have) {
     const int first_q_pos = inf.q_pos + qoff, shift = inf.shift;
-    __syncthreads();   // the previous tile has been read by every wavefront
-    bwd_stash_tile<D>(qt, q_rows, q_tr);
-    bwd_stash_tile<D>(gt, g_rows, g_tr);
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the tile has landed (and its lse, delta)
     if (threadIdx.x < 64) {
-      lse_s[threadIdx.x] = l2_next;
-      dlt_s[threadIdx.x] = dl_next;
+      rowv[buf * 128 + threadIdx.x] = l2_next;
+      rowv[buf * 128 + 64 + threadIdx.x] = dl_next;
     }
-    __syncthreads();
+    __syncthreads();   // ... every wavefront's, and the other buffer has been read by all
+    const char *q_t = lds + buf * 2 * T::TILE_BYTES, *g_t = q_t + T::TILE_BYTES;
+    const float *lse_s = rowv + buf * 128, *dlt_s = lse_s + 64;
     have = next_tile();
-    if (have) fetch();   // on its way while this tile is computed on
+    if (have) fetch(buf ^ 1);   // on its way while this tile is computed on
+    buf ^= 1;
     if (!active) continue;
     // rows of the tile from first_vis on see this lane's key (causal); lanes past the block's keys see nothing
     int first_vis = 0;
     if (p.causal) first_vis = max(0, key_pos - shift - first_q_pos);
     if (l32 >= nrows) first_vis = 64;
-    // With one workgroup per CU (D = 128) registers are plentiful: both halves' S and dP are formed
-    // first, so that the matrix products of one half can overlap the vector work of the other.
-    constexpr bool kEager = D > 64;
-    f32x16 s2[2], dp2[2];
-    if constexpr (kEager) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        s2[h] = bwd_rows_times_frag<D, E>(q_rows, h, kf, lane);
-        dp2[h] = bwd_rows_times_frag<D, E>(g_rows, h, vf, lane);
-      }
-    }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      f32x16 s, dp;
-      if constexpr (kEager) {
-        s = s2[h];
-        dp = dp2[h];
-      } else {
-        s = bwd_rows_times_frag<D, E>(q_rows, h, kf, lane);
-        dp = bwd_rows_times_frag<D, E>(g_rows, h, vf, lane);
-      }
+      if (shared_slots && h != part) continue;   // the slot's other wavefront takes these rows
+      const f32x16 s = bwd_rows_times_frag<D, E>(q_t, h, kf, lane);
+      const f32x16 dp = bwd_rows_times_frag<D, E>(g_t, h, vf, lane);
       float ep[16], ed[16];
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
@@ -512,13 +484,36 @@ __global__ __launch_bounds__(kThreads, D <= 64 ? 2 : 1) void hbsa_bwd_dkv_kernel
       short8v plo, phi, dlo, dhi;
       bwd_pack<E>(ep, plo, phi);
       bwd_pack<E>(ed, dlo, dhi);
-      bwd_transposed_times_packed<D, E>(g_tr, 2 * h, plo, lane, acc_v);
-      bwd_transposed_times_packed<D, E>(g_tr, 2 * h + 1, phi, lane, acc_v);
-      bwd_transposed_times_packed<D, E>(q_tr, 2 * h, dlo, lane, acc_k);
-      bwd_transposed_times_packed<D, E>(q_tr, 2 * h + 1, dhi, lane, acc_k);
+      bwd_transposed_times_packed<D, E>(g_t, 2 * h, plo, lane, acc_v);
+      bwd_transposed_times_packed<D, E>(g_t, 2 * h + 1, phi, lane, acc_v);
+      bwd_transposed_times_packed<D, E>(q_t, 2 * h, dlo, lane, acc_k);
+      bwd_transposed_times_packed<D, E>(q_t, 2 * h + 1, dhi, lane, acc_k);
     }
   }
-  if (active && l32 < nrows) {
+  if (shared_slots) {   // the wavefronts of the lower rows hand their sums to those of the upper rows: [slot][register][lane] floats
+    __syncthreads();
+    float *xch = (float *)lds + (size_t)slot * (2 * T::DT * 16) * 64 + lane;
+    if (part == 1) {
+#pragma unroll
+      for (int dt = 0; dt < T::DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          xch[(dt * 16 + i) * 64] = acc_k[dt][i];
+          xch[((T::DT + dt) * 16 + i) * 64] = acc_v[dt][i];
+        }
+    }
+    __syncthreads();
+    if (part == 0) {
+#pragma unroll
+      for (int dt = 0; dt < T::DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          acc_k[dt][i] += xch[(dt * 16 + i) * 64];
+          acc_v[dt][i] += xch[((T::DT + dt) * 16 + i) * 64];
+        }
+    }
+  }
+  if (part == 0 && active && l32 < nrows) {
     const int64_t row = k0 + kbl * p.kbs + row0 + l32;
     bwd_store_rows<D, E>(p.dk + row * p.dk_s + (int64_t)hk * p.dk_h, acc_k, p.scale, g32);
     bwd_store_rows<D, E>(p.dv + row * p.dv_s + (int64_t)hk * p.dv_h, acc_v, 1.f, g32);
@@ -782,7 +777,7 @@ int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_
   const int64_t rows = (int64_t)dp.total_q * dp.nhead_q;
   hipLaunchKernelGGL((hbsa_bwd_delta_kernel<D, E>), dim3((unsigned)((rows * (D / 8) + 255) / 256)), dim3(256), 0, stream, dp);
   // D = 128: tiles, the rows' lse and delta, K and V of the workgroup; at least the 128 KB of the final exchange
-  const int lds_dq = 4 * T::TILE_BYTES, lds_dkv = D == 128 ? 8 * T::TILE_BYTES + 1024 : 4 * T::TILE_BYTES + 512;
+  const int lds_dq = 4 * T::TILE_BYTES, lds_dkv = D == 128 ? 8 * T::TILE_BYTES + 1024 : 4 * T::TILE_BYTES + 1024;
   if (lds_dkv > 48 * 1024) {
     static thread_local bool raised[kMaxDevices] = {};
     int dev = 0;

@@ -2045,11 +2045,11 @@ int hbsa_bwd(const void *q, const void *k, const void *v, const void *out, const
     return fail(HBSA_ERR_WORKSPACE_TOO_SMALL, "bwd_workspace smaller than hbsa_bwd_workspace_bytes, or not 16-byte aligned");
   if (total_q == 0 || total_k == 0 || num_q_block == 0 || num_k_block == 0) return 0;
   // (the kernels address a tile's rows with 32-bit offsets from the tile's first row: K and V tiles in the dQ
-  // kernel, Q and dO tiles in the D = 128 dK/dV kernel)
+  // kernel, Q and dO tiles in the dK/dV kernels)
   if (strides[2] < 0 || strides[4] < 0 || strides[2] > (1 << 24) || strides[4] > (1 << 24))
     return fail(HBSA_ERR_UNSUPPORTED, "k/v token stride (%lld, %lld elements) outside [0, 2^24]", (long long)strides[2],
                 (long long)strides[4]);
-  if (headdim == 128 && (strides[0] < 0 || strides[8] < 0 || strides[0] > (1 << 24) || strides[8] > (1 << 24)))
+  if (strides[0] < 0 || strides[8] < 0 || strides[0] > (1 << 24) || strides[8] > (1 << 24))
     return fail(HBSA_ERR_UNSUPPORTED, "q/dout token stride (%lld, %lld elements) outside [0, 2^24]", (long long)strides[0],
                 (long long)strides[8]);
 

@@ -18,7 +18,7 @@
  *     through hbsa_last_error(), which is thread-local), positive = hipError_t;
  *   - strides are in ELEMENTS; the innermost (head-dim) stride of q/k/v/out must be 1 and
  *     every row must start on a 16-byte boundary.  The token strides of k and v (and, in the
- *     backward at headdim 128, of q and dout) must lie in [0, 2^24]: the kernels address the
+ *     backward, of q and dout) must lie in [0, 2^24]: the kernels address the
  *     rows of a tile with 32-bit offsets.  Other strides may take any value, negative included.
  */
 #ifndef HBSATTN_AMD_H_
