@@ -520,47 +520,31 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dkv_kernel(BwdParams p) 
   }
 }
 
-// ---- dK, dV at D = 128: eight wavefronts -------------------------------------------------------------
-// The kernel above holds K^T, V^T and both accumulators of a wavefront in registers: 256 + 238 at
-// D = 128, one wavefront per SIMD.  This one keeps the workgroup's K and V rows in LDS (read as B
-// operands per product) and runs eight wavefronts: wavefronts w and w + 4 own the same 32 keys and
-// take rows 0-31 and 32-63 of every tile, so that two wavefronts share a SIMD and cover each other's
-// waits; their two partial accumulators are added through LDS at the end.  No product is computed twice.
-//
-// The Q and dO tiles go from global memory straight into LDS (global_load_lds_dwordx4, 16 bytes per lane
-// to M0 + 16 * lane), two buffers each: tile t + 1 travels while tile t is computed on, one barrier per
-// tile.  A tile is read both by rows (A operand of S and dP) and transposed (A operand of the dK^T, dV^T
-// updates) and is stored once, in the layout of BwdTile::swz_both.
-
-// acc[dt] += tile^T (rows 16*g .. 16*g+15 as the contraction index) . packed, tile in the swz_both layout
-template <typename E>
-__device__ __forceinline__ void dkv8_transposed_times_packed(const char *tile, int g, short8v packed, int rd_lo, int rd_hi, f32x16 *acc) {
-#pragma unroll
-  for (int dt = 0; dt < 4; ++dt) {
-    const char *a = tile + (rd_lo ^ (dt * 64)) + g * 16 * BwdTile<128>::RB;
-    const char *b = tile + (rd_hi ^ (dt * 64)) + g * 16 * BwdTile<128>::RB;
-    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(a));
-    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)HBSA_AS3(b));
-    const short8v va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    acc[dt] = E::mfma(va, packed, acc[dt]);
-  }
-}
-
+// ---- dK, dV at D = 128: eight wavefronts in two roles -------------------------------------------------
+// The kernel above would hold K^T, V^T and both accumulators of a wavefront in registers: 256 + 238 at
+// D = 128, one wavefront per SIMD.  Here two wavefronts share a 32-key slot (and a SIMD) and split the four
+// products between them, each with one operand and one accumulator in registers:
+//   the P wavefront  keeps K^T:  S = Q K^T,  P = exp(S - lse) (masked),   dV^T += dO^T P,   hands P over;
+//   the dS wavefront keeps V^T:  dP = dO V^T,  dS = P * (dP - delta),      dK^T += Q^T dS.
+// P travels through LDS as the packed 16-bit operand the P wavefront feeds to its own product (4 KB per slot
+// and tile), and one tile late: in the iteration in which the P wavefront works on tile t, the dS wavefront
+// finishes tile t - 1 (whose dP it kept in registers) and forms dP of tile t, so one barrier per tile orders
+// everything.  Hence three Q tile buffers (tile t - 1 is still read while tile t + 1 arrives), two for dO.
+// Tiles go from global memory straight into LDS, stored once in the layout of BwdTile::swz_both.
 template <typename E>
 __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   constexpr int D = 128;
   using T = BwdTile<D>;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  // buffer s of the tiles: Q rows at s * 2 * TILE_BYTES, dO rows one tile further (the first 64 KB, which
-  // the M0 offsets of the direct loads can address)
-  char *tiles = lds;
-  float *rowv = (float *)(lds + 4 * T::TILE_BYTES);    // buffer s: [64] log2-domain log-sum-exp of the tile's rows, [64] their delta
-  char *k_blk = lds + 4 * T::TILE_BYTES + 1024;        // [128][D] keys of the workgroup, layout read by rows
-  char *v_blk = k_blk + 2 * T::TILE_BYTES;
+  char *q_buf = lds;                                   // [3] Q tiles
+  char *g_buf = lds + 3 * T::TILE_BYTES;               // [2] dO tiles
+  char *p_buf = lds + 5 * T::TILE_BYTES;               // [2 tile parities][4 slots][2 halves][lo, hi][64 lanes] 16 bytes
+  float *lse_s = (float *)(lds + 7 * T::TILE_BYTES);   // [2][64] log2-domain log-sum-exp of the tile's rows
+  float *dlt_s = lse_s + 128;                          // [3][64] their delta
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int slot = wave & 3, half = wave >> 2;   // 32-key slot of the workgroup; which 32 rows of a tile
+  const int slot = wave & 3, role = wave >> 2;   // 32-key slot of the workgroup; 0: the P wavefront, 1: the dS wavefront
   const int g32 = lane >> 5, l32 = lane & 31;
   // With a multiple of eight kv heads the grid is one-dimensional and workgroup ids, which go round the
   // eight XCDs (each with its own L2), are decoded so that XCD x works on the heads x, x + 8, ...: the
@@ -590,25 +574,23 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   const int key_pos = kbl * p.kbs + min(row0 + l32, krows - 1);
   const int wg_first_key = kbl * p.kbs + wg_row0;
 
-  // the workgroup's 128 key rows (rows past the block's end repeat its last key; their lanes are masked)
-  {
-    const char *kbase = p.k + (int64_t)(k0 + kbl * p.kbs) * p.k_s + (int64_t)hk * p.k_h;
-    const char *vbase = p.v + (int64_t)(k0 + kbl * p.kbs) * p.v_s + (int64_t)hk * p.v_h;
+  // this wavefront's resident operand: K^T (P wavefront) or V^T (dS wavefront) of its 32 keys; lane holds
+  // key l32, d = 16 * ks + 8 * g32 .. + 7
+  short8v frag[T::KSTEPS];
+  if (active) {
+    const char *src = role == 0 ? p.k + (int64_t)(k0 + key_pos) * p.k_s + (int64_t)hk * p.k_h
+                                : p.v + (int64_t)(k0 + key_pos) * p.v_s + (int64_t)hk * p.v_h;
 #pragma unroll
-    for (int i = 0; i < 128 * T::CPR / 512; ++i) {
-      const int ch = i * 512 + threadIdx.x;
-      const int r = ch / T::CPR, pc = ch % T::CPR;
-      const int64_t src_row = min(wg_row0 + r, krows - 1);
-      const int dst = r * T::RB + ((pc ^ T::swz_rows(r)) << 4);
-      *(u32x4 *)(k_blk + dst) = *(const u32x4 *)(kbase + src_row * p.k_s + pc * 16);
-      *(u32x4 *)(v_blk + dst) = *(const u32x4 *)(vbase + src_row * p.v_s + pc * 16);
-    }
+    for (int ks = 0; ks < T::KSTEPS; ++ks) frag[ks] = *(const short8v *)(src + g32 * 16 + ks * 32);
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < T::KSTEPS; ++ks) frag[ks] = short8v{0, 0, 0, 0, 0, 0, 0, 0};
   }
-  f32x16 acc_k[T::DT], acc_v[T::DT];
+  f32x16 acc[T::DT];   // dV^T (P wavefront) or dK^T (dS wavefront) of the 32 keys
 #pragma unroll
   for (int dt = 0; dt < T::DT; ++dt)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { acc_k[dt][i] = 0.f; acc_v[dt][i] = 0.f; }
+    for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
 
   int qb = p.cu_num_q_block[b] - 1, r = 0, qoff = 0;
   const int qb_end = p.cu_num_q_block[b + 1];
@@ -655,26 +637,26 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   };
   // A tile's 1024 chunks over eight wavefronts: wavefront w fills rows 4 * (8 * i + w) .. + 3 with load i
   // (i = 0, 1), lane l the 16 bytes at chunk position l % 16 of row l / 16 of those, which hold the
-  // row's chunk (l % 16) ^ swz(row).
+  // row's chunk (l % 16) ^ swz_both(row).
   const int ld_row = 4 * wave + (lane >> 4);                              // + 32 * i
   const uint32_t ld_chunk = (uint32_t)(((lane & 15) ^ T::swz_both(ld_row & 15)) * 16);
   const uint32_t q_s32 = (uint32_t)p.q_s, do_s32 = (uint32_t)p.do_s;      // the host checks that they fit
-  const uint32_t tiles_addr = (uint32_t)(uintptr_t)HBSA_AS3(tiles) + (uint32_t)wave * 1024u;
+  const uint32_t q_addr = (uint32_t)(uintptr_t)HBSA_AS3(q_buf) + (uint32_t)wave * 1024u;
+  const uint32_t g_addr = (uint32_t)(uintptr_t)HBSA_AS3(g_buf) + (uint32_t)wave * 1024u;
   float l2_next = INFINITY, dl_next = 0.f;
-  auto fetch = [&](int buf) {
+  auto fetch = [&](int qi, int gi) {   // the tile next_tile() has moved to, into Q buffer qi and dO buffer gi
     const int valid = min(64, inf.rows - qoff);
     const int64_t row_first = inf.row_begin + qoff;
     const int hq = hk * p.ratio + r;
     const char *qsrc = p.q + row_first * p.q_s + (int64_t)hq * p.q_h;
     const char *gsrc = p.dout + row_first * p.do_s + (int64_t)hq * p.do_h;
-    const uint32_t dst = tiles_addr + (uint32_t)(buf * 2 * T::TILE_BYTES);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const uint32_t rr = (uint32_t)min(ld_row + 32 * i, valid - 1);   // rows past the block's end repeat its last row
-      bwd_dma16(dst + (uint32_t)(i * 8 * 1024), qsrc, rr * q_s32 + ld_chunk);
-      bwd_dma16(dst + (uint32_t)(T::TILE_BYTES + i * 8 * 1024), gsrc, rr * do_s32 + ld_chunk);
+      bwd_dma16(q_addr + (uint32_t)(qi * T::TILE_BYTES + i * 8 * 1024), qsrc, rr * q_s32 + ld_chunk);
+      bwd_dma16(g_addr + (uint32_t)(gi * T::TILE_BYTES + i * 8 * 1024), gsrc, rr * do_s32 + ld_chunk);
     }
-    l2_next = INFINITY;
+    l2_next = INFINITY;   // rows past the block's end take no part: P = exp2(-inf) = 0
     dl_next = 0.f;
     if (threadIdx.x < valid) {
       const float l = p.lse[(row_first + threadIdx.x) * p.nhead_q + hq];
@@ -682,93 +664,110 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
       dl_next = p.delta[(row_first + threadIdx.x) * p.nhead_q + hq];
     }
   };
-  // this lane's operand reads: by rows (16 bytes of row l32, k-step 0) and transposed (keys 0-7 and 8-15 of a group)
-  const int rd = l32 * T::RB + ((g32 ^ T::swz_both(l32 & 15)) << 4);
-  const int rd_b = l32 * T::RB + ((g32 ^ T::swz_rows(l32)) << 4);   // K and V rows of the workgroup
-  const int tr_key = 4 * g32 + ((lane & 15) >> 2);
-  const int tr_lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-  const int rd_lo = tr_key * T::RB + ((tr_lc ^ T::swz_both(tr_key)) << 4) + 8 * (lane & 1);
-  const int rd_hi = (tr_key + 8) * T::RB + ((tr_lc ^ T::swz_both(tr_key + 8)) << 4) + 8 * (lane & 1);
+  // this lane's 32 bytes of a (tile parity, slot, half) record of P
+  char *p_mine = p_buf + (size_t)slot * 4096 + lane * 16;
 
-  bool have = next_tile();
-  int buf = 0;
-  if (have) fetch(0);
-  while (have) {
-    const int first_q_pos = inf.q_pos + qoff, shift = inf.shift;
-    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the tile has landed (and its lse, delta)
-    if (threadIdx.x < 64) {
-      rowv[buf * 128 + threadIdx.x] = l2_next;
-      rowv[buf * 128 + 64 + threadIdx.x] = dl_next;
+  // The loop exists once per role (the same barriers in both): with the roles as branches of one loop body the
+  // register allocator keeps both roles' temporaries apart and spills.
+  auto run = [&](auto role_) {
+  constexpr int ROLE = decltype(role_)::value;
+  bool cur = next_tile();   // a tile for this iteration
+  bool prev = false;        // the tile before it exists: its dK part is still due
+  int qi = 0, par = 0;      // Q buffer (of three) and parity of the current tile
+  f32x16 dp_prev[2];        // dS wavefront: dP of the previous tile, both halves
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dp_prev[h][i] = 0.f;
+  if (cur) fetch(0, 0);
+  while (cur || prev) {
+    const int first_q_pos = inf.q_pos + qoff, shift = inf.shift;   // of the current tile (if any)
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the current tile has landed (and its lse, delta)
+    if (cur && threadIdx.x < 64) {
+      lse_s[par * 64 + threadIdx.x] = l2_next;
+      dlt_s[qi * 64 + threadIdx.x] = dl_next;
     }
-    __syncthreads();   // ... every wavefront's; the other buffer has been read by all (and, the first time, K and V are in place)
-    const char *q_t = tiles + buf * 2 * T::TILE_BYTES, *g_t = q_t + T::TILE_BYTES;
-    const float *lse_s = rowv + buf * 128, *dlt_s = lse_s + 64;
-    have = next_tile();
-    if (have) fetch(buf ^ 1);
-    buf ^= 1;
-    if (!active) continue;
-    int first_vis = 0;
-    if (p.causal) first_vis = max(0, key_pos - shift - first_q_pos);
-    if (l32 >= nrows) first_vis = 64;
-    // rows 32*half .. +31 of the tile against this wavefront's 32 keys
-    f32x16 sv, dp;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) { sv[i] = 0.f; dp[i] = 0.f; }
-#pragma unroll
-    for (int ks = 0; ks < T::KSTEPS; ++ks) {
-      const int a_off = (rd ^ (ks * 32)) + half * 32 * T::RB, b_off = (rd_b ^ (ks * 32)) + slot * 32 * T::RB;
-      sv = E::mfma(*(const short8v *)(q_t + a_off), *(const short8v *)(k_blk + b_off), sv);
-      dp = E::mfma(*(const short8v *)(g_t + a_off), *(const short8v *)(v_blk + b_off), dp);
+    __syncthreads();   // ... every wavefront's; what the iteration before read and wrote is settled
+    const int q_now = qi, q_before = qi == 0 ? 2 : qi - 1, q_after = qi == 2 ? 0 : qi + 1;
+    const bool had = cur;
+    if (cur) {
+      cur = next_tile();
+      if (cur) fetch(q_after, par ^ 1);   // on its way during this iteration (the buffers it fills were last read an iteration ago)
     }
-    float ep[16], ed[16];
+    if (active) {
+      if constexpr (ROLE == 0) {
+        if (had) {   // ---- P wavefront, current tile
+          const char *q_t = q_buf + q_now * T::TILE_BYTES, *g_t = g_buf + par * T::TILE_BYTES;
+          int first_vis = 0;   // rows of the tile from first_vis on see this lane's key (causal)
+          if (p.causal) first_vis = max(0, key_pos - shift - first_q_pos);
+          if (l32 >= nrows) first_vis = 64;
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      const int rr0 = 32 * half + 8 * a + 4 * g32;
-      const f32x4 l4 = *(const f32x4 *)(lse_s + rr0), d4 = *(const f32x4 *)(dlt_s + rr0);
+          for (int h = 0; h < 2; ++h) {
+            const f32x16 sv = bwd_rows_times_frag<D, E>(q_t, h, frag, lane);
+            float ep[16];
 #pragma unroll
-      for (int bq = 0; bq < 4; ++bq) {
-        const int i = 4 * a + bq;
-        const bool vis = rr0 + bq >= first_vis;   // rows past the block's end carry lse = +inf, hence P = 0
-        const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(sv[i], p.c, -l4[bq])) : 0.f;
-        ep[i] = pv;
-        ed[i] = pv * (dp[i] - d4[bq]);
+            for (int a = 0; a < 4; ++a) {
+              const int rr0 = 32 * h + 8 * a + 4 * g32;
+              const f32x4 l4 = *(const f32x4 *)(lse_s + par * 64 + rr0);
+#pragma unroll
+              for (int bq = 0; bq < 4; ++bq) {
+                const bool vis = rr0 + bq >= first_vis;   // rows past the block's end carry lse = +inf, hence P = 0
+                ep[4 * a + bq] = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(sv[4 * a + bq], p.c, -l4[bq])) : 0.f;
+              }
+            }
+            short8v plo, phi;
+            bwd_pack<E>(ep, plo, phi);
+            *(short8v *)(p_mine + par * 16384 + h * 2048) = plo;
+            *(short8v *)(p_mine + par * 16384 + h * 2048 + 1024) = phi;
+            bwd_transposed_times_packed<D, E>(g_t, 2 * h, plo, lane, acc);
+            bwd_transposed_times_packed<D, E>(g_t, 2 * h + 1, phi, lane, acc);
+          }
+        }
+      } else {
+        if (prev) {   // ---- dS wavefront, the tile before: dS = P * (dP - delta), dK^T += Q^T dS
+          const char *q_t = q_buf + q_before * T::TILE_BYTES;
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const u32x4 wlo = *(const u32x4 *)(p_mine + (par ^ 1) * 16384 + h * 2048);
+            const u32x4 whi = *(const u32x4 *)(p_mine + (par ^ 1) * 16384 + h * 2048 + 1024);
+            float ed[16];
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+              const int rr0 = 32 * h + 8 * a + 4 * g32;
+              const f32x4 d4 = *(const f32x4 *)(dlt_s + q_before * 64 + rr0);
+#pragma unroll
+              for (int bq = 0; bq < 4; ++bq) {
+                const int i = 4 * a + bq;
+                const uint32_t w = (i < 8 ? wlo : whi)[(i & 7) >> 1];
+                const float pv = (i & 1) ? E::hi(w) : E::lo(w);
+                ed[i] = pv * (dp_prev[h][i] - d4[bq]);
+              }
+            }
+            short8v dlo, dhi;
+            bwd_pack<E>(ed, dlo, dhi);
+            bwd_transposed_times_packed<D, E>(q_t, 2 * h, dlo, lane, acc);
+            bwd_transposed_times_packed<D, E>(q_t, 2 * h + 1, dhi, lane, acc);
+          }
+        }
+        if (had) {   // ---- dS wavefront, current tile: dP = dO V^T, kept for the next iteration
+          const char *g_t = g_buf + par * T::TILE_BYTES;
+#pragma unroll
+          for (int h = 0; h < 2; ++h) dp_prev[h] = bwd_rows_times_frag<D, E>(g_t, h, frag, lane);
+        }
       }
     }
-    short8v plo, phi, dlo, dhi;
-    bwd_pack<E>(ep, plo, phi);
-    bwd_pack<E>(ed, dlo, dhi);
-    dkv8_transposed_times_packed<E>(g_t, 2 * half, plo, rd_lo, rd_hi, acc_v);
-    dkv8_transposed_times_packed<E>(g_t, 2 * half + 1, phi, rd_lo, rd_hi, acc_v);
-    dkv8_transposed_times_packed<E>(q_t, 2 * half, dlo, rd_lo, rd_hi, acc_k);
-    dkv8_transposed_times_packed<E>(q_t, 2 * half + 1, dhi, rd_lo, rd_hi, acc_k);
+    prev = had;
+    qi = q_after;
+    par ^= 1;
   }
-  // wavefronts 4-7 hand their partial sums to wavefronts 0-3 through LDS: [slot][register][lane] floats
-  __syncthreads();
-  float *xch = (float *)lds + (size_t)slot * 128 * 64 + lane;
-  if (half == 1) {
-#pragma unroll
-    for (int dt = 0; dt < T::DT; ++dt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        xch[(dt * 16 + i) * 64] = acc_k[dt][i];
-        xch[(64 + dt * 16 + i) * 64] = acc_v[dt][i];
-      }
+  if (active && l32 < nrows) {
+    const int64_t row = k0 + kbl * p.kbs + row0 + l32;
+    if constexpr (ROLE == 0) bwd_store_rows<D, E>(p.dv + row * p.dv_s + (int64_t)hk * p.dv_h, acc, 1.f, g32);
+    else bwd_store_rows<D, E>(p.dk + row * p.dk_s + (int64_t)hk * p.dk_h, acc, p.scale, g32);
   }
-  __syncthreads();
-  if (half == 0 && active) {
-#pragma unroll
-    for (int dt = 0; dt < T::DT; ++dt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        acc_k[dt][i] += xch[(dt * 16 + i) * 64];
-        acc_v[dt][i] += xch[(64 + dt * 16 + i) * 64];
-      }
-    if (l32 < nrows) {
-      const int64_t row = k0 + kbl * p.kbs + row0 + l32;
-      bwd_store_rows<D, E>(p.dk + row * p.dk_s + (int64_t)hk * p.dk_h, acc_k, p.scale, g32);
-      bwd_store_rows<D, E>(p.dv + row * p.dv_s + (int64_t)hk * p.dv_h, acc_v, 1.f, g32);
-    }
-  }
+  };
+  if (role == 0) run(std::integral_constant<int, 0>{});
+  else run(std::integral_constant<int, 1>{});
 }
 
 template <int D, typename E>
@@ -777,7 +776,7 @@ int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_
   const int64_t rows = (int64_t)dp.total_q * dp.nhead_q;
   hipLaunchKernelGGL((hbsa_bwd_delta_kernel<D, E>), dim3((unsigned)((rows * (D / 8) + 255) / 256)), dim3(256), 0, stream, dp);
   // D = 128: tiles, the rows' lse and delta, K and V of the workgroup; at least the 128 KB of the final exchange
-  const int lds_dq = 4 * T::TILE_BYTES, lds_dkv = D == 128 ? 8 * T::TILE_BYTES + 1024 : 4 * T::TILE_BYTES + 1024;
+  const int lds_dq = 4 * T::TILE_BYTES, lds_dkv = D == 128 ? 7 * T::TILE_BYTES + 2048 : 4 * T::TILE_BYTES + 1024;
   if (lds_dkv > 48 * 1024) {
     static thread_local bool raised[kMaxDevices] = {};
     int dev = 0;
