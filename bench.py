@@ -167,6 +167,11 @@ def measure(name, steps, warmup):
                            "kernel": "hbsa_fwd_kernel", "kernel_ms": kernel_ms, "algorithmic_bytes": work["bytes"],
                            "flop_per_byte": intensity,
                            "mfma_frac": work["flops"] / kernel_ms / 1e9 / PEAK_BF16_TFLOPS}
+    if traffic is not None:
+        # the profiled HBM bytes per launch over this run's kernel time: how much of the 8 TB/s the kernel's
+        # actual traffic (re-reads of K/V blocks included) takes, whatever roof the algorithmic figures name
+        res["roofline"]["traffic_gb_s"] = traffic / kernel_ms / 1e6
+        res["roofline"]["traffic_frac_of_hbm_peak"] = traffic / kernel_ms / 1e6 / PEAK_HBM_GBS
     return w, res
 
 
