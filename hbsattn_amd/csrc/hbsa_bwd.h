@@ -526,8 +526,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dkv_kernel(BwdParams p) 
 // products between them, each with one operand and one accumulator in registers:
 //   the P wavefront  keeps K^T:  S = Q K^T,  P = exp(S - lse) (masked),   dV^T += dO^T P,   hands P over;
 //   the dS wavefront keeps V^T:  dP = dO V^T,  dS = P * (dP - delta),      dK^T += Q^T dS.
-// P travels through LDS as the packed 16-bit operand the P wavefront feeds to its own product (4 KB per slot
-// and tile), and one tile late: in the iteration in which the P wavefront works on tile t, the dS wavefront
+// P travels through LDS in fp32 (8 KB per slot and tile; dS is formed from the unrounded P), and one tile late: in the iteration in which the P wavefront works on tile t, the dS wavefront
 // finishes tile t - 1 (whose dP it kept in registers) and forms dP of tile t, so one barrier per tile orders
 // everything.  Hence three Q tile buffers (tile t - 1 is still read while tile t + 1 arrives), two for dO.
 // Tiles go from global memory straight into LDS, stored once in the layout of BwdTile::swz_both.
@@ -538,8 +537,8 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   char *q_buf = lds;                                   // [3] Q tiles
   char *g_buf = lds + 3 * T::TILE_BYTES;               // [2] dO tiles
-  char *p_buf = lds + 5 * T::TILE_BYTES;               // [2 tile parities][4 slots][2 halves][lo, hi][64 lanes] 16 bytes
-  float *lse_s = (float *)(lds + 7 * T::TILE_BYTES);   // [2][64] log2-domain log-sum-exp of the tile's rows
+  char *p_buf = lds + 5 * T::TILE_BYTES;               // [2 tile parities][4 slots][2 halves][4][64 lanes] four floats
+  float *lse_s = (float *)(lds + 9 * T::TILE_BYTES);   // [2][64] log2-domain log-sum-exp of the tile's rows
   float *dlt_s = lse_s + 128;                          // [3][64] their delta
 
   const int lane = threadIdx.x & 63;
@@ -664,8 +663,8 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
       dl_next = p.delta[(row_first + threadIdx.x) * p.nhead_q + hq];
     }
   };
-  // this lane's 32 bytes of a (tile parity, slot, half) record of P
-  char *p_mine = p_buf + (size_t)slot * 4096 + lane * 16;
+  // this lane's 4 x 16 bytes of a (tile parity, slot, half) record of P
+  char *p_mine = p_buf + (size_t)slot * 8192 + lane * 16;
 
   // The loop exists once per role (the same barriers in both): with the roles as branches of one loop body the
   // register allocator keeps both roles' temporaries apart and spills.
@@ -715,10 +714,11 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
                 ep[4 * a + bq] = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(sv[4 * a + bq], p.c, -l4[bq])) : 0.f;
               }
             }
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+              *(f32x4 *)(p_mine + par * 32768 + h * 4096 + a * 1024) = f32x4{ep[4 * a], ep[4 * a + 1], ep[4 * a + 2], ep[4 * a + 3]};
             short8v plo, phi;
             bwd_pack<E>(ep, plo, phi);
-            *(short8v *)(p_mine + par * 16384 + h * 2048) = plo;
-            *(short8v *)(p_mine + par * 16384 + h * 2048 + 1024) = phi;
             bwd_transposed_times_packed<D, E>(g_t, 2 * h, plo, lane, acc);
             bwd_transposed_times_packed<D, E>(g_t, 2 * h + 1, phi, lane, acc);
           }
@@ -728,20 +728,14 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
           const char *q_t = q_buf + q_before * T::TILE_BYTES;
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
-            const u32x4 wlo = *(const u32x4 *)(p_mine + (par ^ 1) * 16384 + h * 2048);
-            const u32x4 whi = *(const u32x4 *)(p_mine + (par ^ 1) * 16384 + h * 2048 + 1024);
             float ed[16];
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
               const int rr0 = 32 * h + 8 * a + 4 * g32;
               const f32x4 d4 = *(const f32x4 *)(dlt_s + q_before * 64 + rr0);
+              const f32x4 p4 = *(const f32x4 *)(p_mine + (par ^ 1) * 32768 + h * 4096 + a * 1024);
 #pragma unroll
-              for (int bq = 0; bq < 4; ++bq) {
-                const int i = 4 * a + bq;
-                const uint32_t w = (i < 8 ? wlo : whi)[(i & 7) >> 1];
-                const float pv = (i & 1) ? E::hi(w) : E::lo(w);
-                ed[i] = pv * (dp_prev[h][i] - d4[bq]);
-              }
+              for (int bq = 0; bq < 4; ++bq) ed[4 * a + bq] = p4[bq] * (dp_prev[h][4 * a + bq] - d4[bq]);
             }
             short8v dlo, dhi;
             bwd_pack<E>(ed, dlo, dhi);
@@ -776,7 +770,7 @@ int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_
   const int64_t rows = (int64_t)dp.total_q * dp.nhead_q;
   hipLaunchKernelGGL((hbsa_bwd_delta_kernel<D, E>), dim3((unsigned)((rows * (D / 8) + 255) / 256)), dim3(256), 0, stream, dp);
   // D = 128: tiles, the rows' lse and delta, K and V of the workgroup; at least the 128 KB of the final exchange
-  const int lds_dq = 4 * T::TILE_BYTES, lds_dkv = D == 128 ? 7 * T::TILE_BYTES + 2048 : 4 * T::TILE_BYTES + 1024;
+  const int lds_dq = 4 * T::TILE_BYTES, lds_dkv = D == 128 ? 9 * T::TILE_BYTES + 2048 : 4 * T::TILE_BYTES + 1024;
   if (lds_dkv > 48 * 1024) {
     static thread_local bool raised[kMaxDevices] = {};
     int dev = 0;
