@@ -176,7 +176,7 @@ def measure(name, steps, warmup):
 
 
 def measure_backward(w, flops, steps):
-    """Device time of one backward call (delta, dq and dk/dv kernels) for the workload's tensors, with
+    """Device time of one backward call (dq and dk/dv kernels) for the workload's tensors, with
     event pairs on the launch stream; FLOPs counted as 2.5 x the forward's over kept blocks."""
     from hbsattn_amd.interface import hbsa_backward, hbsa_prepare, hbsa_run
 
@@ -189,7 +189,7 @@ def measure_backward(w, flops, steps):
         step()
     ms = time_kernel_events(step, steps)
     return {"ms_per_call": ms, "tflops": 2.5 * flops / ms / 1e9, "flops_counted": "2.5 x forward FLOPs over kept blocks",
-            "kernels": "hbsa_bwd_delta_kernel + hbsa_bwd_dq_kernel + hbsa_bwd_dkv8_kernel (hbsa_bwd_dkv_kernel below D=128)"}
+            "kernels": "hbsa_bwd_dq_kernel + hbsa_bwd_dkv8_kernel (hbsa_bwd_dkv_kernel below D=128)"}
 
 
 def cpu_baseline(w, budget_s=20.0):

@@ -8,13 +8,14 @@
 //     dV = P^T dO      dP = dO V^T      dS = P * (dP - delta)
 //     dQ = scale * dS K                 dK = scale * dS^T Q
 //
-// Three launches per call, no atomics, every output element written by exactly one workgroup:
-//   hbsa_bwd_delta_kernel : delta[row, q head] = sum_d dO * O
+// Two launches per call, no atomics, every output element written by exactly one workgroup:
 //   hbsa_bwd_dq_kernel    : one workgroup per (kv head, q block, group of four 32-row wave slots), the
 //                           forward's decomposition; walks the kept k blocks of the q block's bit row.
 //                           Per 64-key tile  S^T = K Q^T,  dP^T = V dO^T  (A = tile rows from LDS,
 //                           B = Q^T / dO^T in registers),  dS^T in the accumulator layout is the B
-//                           operand of  dQ^T += K^T dS^T  (A = K^T through transposing LDS reads).
+//                           operand of  dQ^T += K^T dS^T  (A = K^T through transposing LDS reads).  It also forms
+//                           delta of its rows (it holds their dO; their O is one more row load) and leaves
+//                           it for the second launch.
 //   hbsa_bwd_dkv_kernel   : (head dims up to 64; hbsa_bwd_dkv8_kernel is the form for D = 128) the same
 //                           with the roles of queries and keys exchanged: one workgroup per
 //                           (kv head, k block, group of four 32-key slots); K^T and V^T stay in
@@ -30,50 +31,20 @@
 namespace {
 
 struct BwdParams {
-  const char *q, *k, *v, *dout;
+  const char *q, *k, *v, *out, *dout;
   char *dq, *dk, *dv;
-  const float *lse, *delta;   // [total_q, nhead_q], contiguous
+  const float *lse;           // [total_q, nhead_q], contiguous
+  float *delta;               // [total_q, nhead_q], contiguous: rowsum(dO * O), written by the dQ kernel, read by the dK/dV kernels
   const QBlockInfo *info;
   const uint32_t *bits;
   const int32_t *cu_k, *cu_num_q_block, *cu_num_k_block;
-  int64_t q_s, q_h, k_s, k_h, v_s, v_h, do_s, do_h, dq_s, dq_h, dk_s, dk_h, dv_s, dv_h;   // bytes
+  int64_t q_s, q_h, k_s, k_h, v_s, v_h, o_s, o_h, do_s, do_h, dq_s, dq_h, dk_s, dk_h, dv_s, dv_h;   // bytes
   int32_t nqb, nkb, xcd_heads, batch, ratio, nhead_q, qbs, kbs, wpr, causal;   // xcd_heads: see the dK/dV kernels
   int32_t wps, nsub;     // q side: wave slots per q head and workgroups per (kv head, q block), as in the forward
   int32_t nsub_k;        // k side: workgroups per (kv head, k block) = ceil(k_block_size / 128)
   float c;               // softmax_scale * log2(e), signed
   float scale;
 };
-
-struct DeltaParams {
-  const char *out, *dout;
-  float *delta;
-  int64_t o_s, o_h, do_s, do_h;   // bytes
-  int32_t total_q, nhead_q;
-};
-
-// delta[row, head] = sum over d of dO * O; D/8 neighbouring lanes share a (row, head), 16 bytes each
-template <int D, typename E>
-__global__ __launch_bounds__(256) void hbsa_bwd_delta_kernel(DeltaParams p) {
-  constexpr int LPR = D / 8;   // lanes per row: 4, 8 or 16
-  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LPR;
-  const int ch = threadIdx.x % LPR;
-  const bool live = i < (int64_t)p.total_q * p.nhead_q;
-  float acc = 0.f;
-  if (live) {
-    const int64_t row = i / p.nhead_q;
-    const int h = (int)(i - row * p.nhead_q);
-    const u32x4 a = *(const u32x4 *)(p.out + row * p.o_s + h * p.o_h + ch * 16);
-    const u32x4 b = *(const u32x4 *)(p.dout + row * p.do_s + h * p.do_h + ch * 16);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      acc += E::lo(a[j]) * E::lo(b[j]);
-      acc += E::hi(a[j]) * E::hi(b[j]);
-    }
-  }
-#pragma unroll
-  for (int m = LPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m);
-  if (live && ch == 0) p.delta[i] = acc;
-}
 
 // ---- shared pieces of the two main kernels ---------------------------------------------------------
 template <int D>
@@ -209,7 +180,20 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
     }
     const float l = p.lse[(int64_t)my_row * p.nhead_q + hq];
     lse2 = l == -INFINITY ? INFINITY : l * kLog2e;
-    dlt = p.delta[(int64_t)my_row * p.nhead_q + hq];
+    // delta = sum over d of dO * O of the row: this lane's half of the head dim, then the other half's from lane + 32.
+    // Every (row, q head) belongs to exactly one wavefront of this grid, which also leaves it for the dK/dV kernel.
+    const char *orow = p.out + (int64_t)my_row * p.o_s + (int64_t)hq * p.o_h + g32 * 16;
+#pragma unroll
+    for (int ks = 0; ks < T::KSTEPS; ++ks) {
+      const u32x4 a = __builtin_bit_cast(u32x4, dof[ks]), b = *(const u32x4 *)(orow + ks * 32);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        dlt += E::lo(a[j]) * E::lo(b[j]);
+        dlt += E::hi(a[j]) * E::hi(b[j]);
+      }
+    }
+    dlt = half_sum(dlt);
+    if (g32 == 0 && l32 < nrows) p.delta[(int64_t)my_row * p.nhead_q + hq] = dlt;
   } else {
 #pragma unroll
     for (int ks = 0; ks < T::KSTEPS; ++ks) { qf[ks] = short8v{0, 0, 0, 0, 0, 0, 0, 0}; dof[ks] = qf[ks]; }
@@ -765,11 +749,9 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
 }
 
 template <int D, typename E>
-int launch_bwd(const BwdParams &bp, const DeltaParams &dp, int nhead_k, int num_k_block, hipStream_t stream) {
+int launch_bwd(const BwdParams &bp, int nhead_k, int num_k_block, hipStream_t stream) {
   using T = BwdTile<D>;
-  const int64_t rows = (int64_t)dp.total_q * dp.nhead_q;
-  hipLaunchKernelGGL((hbsa_bwd_delta_kernel<D, E>), dim3((unsigned)((rows * (D / 8) + 255) / 256)), dim3(256), 0, stream, dp);
-  // D = 128: tiles, the rows' lse and delta, K and V of the workgroup; at least the 128 KB of the final exchange
+  // LDS: the dQ kernel's two K/V tile pairs; the dK/dV kernels' tile buffers, P records and row values
   const int lds_dq = 4 * T::TILE_BYTES, lds_dkv = D == 128 ? 9 * T::TILE_BYTES + 2048 : 4 * T::TILE_BYTES + 1024;
   if (lds_dkv > 48 * 1024) {
     static thread_local bool raised[kMaxDevices] = {};

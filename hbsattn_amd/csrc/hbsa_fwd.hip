@@ -2056,14 +2056,15 @@ int hbsa_bwd(const void *q, const void *k, const void *v, const void *out, const
   const int es = 2;
   BwdParams bp;
   std::memset(&bp, 0, sizeof(bp));
-  bp.q = (const char *)q; bp.k = (const char *)k; bp.v = (const char *)v; bp.dout = (const char *)dout;
+  bp.q = (const char *)q; bp.k = (const char *)k; bp.v = (const char *)v; bp.out = (const char *)out; bp.dout = (const char *)dout;
   bp.dq = (char *)dq; bp.dk = (char *)dk; bp.dv = (char *)dv;
-  bp.lse = lse; bp.delta = (const float *)bwd_workspace;
+  bp.lse = lse; bp.delta = (float *)bwd_workspace;
   bp.info = (const QBlockInfo *)workspace;
   bp.bits = (const uint32_t *)((const char *)workspace + bits_offset(nhead_k, num_q_block));
   bp.cu_k = cu_k_seqlens; bp.cu_num_q_block = cu_num_q_block; bp.cu_num_k_block = cu_num_k_block;
   bp.q_s = strides[0] * es; bp.q_h = strides[1] * es; bp.k_s = strides[2] * es; bp.k_h = strides[3] * es;
-  bp.v_s = strides[4] * es; bp.v_h = strides[5] * es; bp.do_s = strides[8] * es; bp.do_h = strides[9] * es;
+  bp.v_s = strides[4] * es; bp.v_h = strides[5] * es; bp.o_s = strides[6] * es; bp.o_h = strides[7] * es;
+  bp.do_s = strides[8] * es; bp.do_h = strides[9] * es;
   bp.dq_s = strides[10] * es; bp.dq_h = strides[11] * es; bp.dk_s = strides[12] * es; bp.dk_h = strides[13] * es;
   bp.dv_s = strides[14] * es; bp.dv_h = strides[15] * es;
   bp.nqb = num_q_block; bp.nkb = num_k_block; bp.batch = batch;
@@ -2077,16 +2078,12 @@ int hbsa_bwd(const void *q, const void *k, const void *v, const void *out, const
                   (long long)num_q_block * bp.nsub * nhead_k < (1LL << 31)) ? 1 : 0;
   bp.c = softmax_scale * kLog2e;
   bp.scale = softmax_scale;
-  DeltaParams dp;
-  dp.out = (const char *)out; dp.dout = (const char *)dout; dp.delta = (float *)bwd_workspace;
-  dp.o_s = strides[6] * es; dp.o_h = strides[7] * es; dp.do_s = strides[8] * es; dp.do_h = strides[9] * es;
-  dp.total_q = total_q; dp.nhead_q = nhead_q;
   hipStream_t st = (hipStream_t)stream;
   const bool bf = dtype == HBSA_DTYPE_BF16;
   switch (headdim) {
-    case 32: return bf ? launch_bwd<32, ElemBF16>(bp, dp, nhead_k, num_k_block, st) : launch_bwd<32, ElemF16>(bp, dp, nhead_k, num_k_block, st);
-    case 64: return bf ? launch_bwd<64, ElemBF16>(bp, dp, nhead_k, num_k_block, st) : launch_bwd<64, ElemF16>(bp, dp, nhead_k, num_k_block, st);
-    default: return bf ? launch_bwd<128, ElemBF16>(bp, dp, nhead_k, num_k_block, st) : launch_bwd<128, ElemF16>(bp, dp, nhead_k, num_k_block, st);
+    case 32: return bf ? launch_bwd<32, ElemBF16>(bp, nhead_k, num_k_block, st) : launch_bwd<32, ElemF16>(bp, nhead_k, num_k_block, st);
+    case 64: return bf ? launch_bwd<64, ElemBF16>(bp, nhead_k, num_k_block, st) : launch_bwd<64, ElemF16>(bp, nhead_k, num_k_block, st);
+    default: return bf ? launch_bwd<128, ElemBF16>(bp, nhead_k, num_k_block, st) : launch_bwd<128, ElemF16>(bp, nhead_k, num_k_block, st);
   }
 }
 }  // extern "C"
