@@ -24,7 +24,8 @@
 //                           S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS.
 // Both recompute S.  The kept blocks of a mask row or column are found with one load per 32 or 64
 // blocks, not one per block.  Tiles go from global memory straight into LDS (global_load_lds_dwordx4),
-// two buffers: tile t + 1 travels while tile t is computed on, one barrier per tile.  A tile that is
+// two buffers (three for the Q tiles of the D = 128 dK/dV kernel): tile t + 1 travels while tile t is computed
+// on, one barrier per tile.  A tile that is
 // read both by rows and transposed is stored once, in a layout without bank conflicts for either
 // (BwdTile::swz_both).  The forward's persistent scheduling is not applied here.
 
@@ -55,10 +56,8 @@ struct BwdTile {
   static constexpr int TILE_BYTES = 64 * RB;
   static constexpr int KSTEPS = D / 16;
   static constexpr int DT = D / 32;
-  // chunk swizzles of the forward's K tile (read by rows) and V tile (read transposed)
-  static __device__ __forceinline__ int swz_rows(int r) { return (r / RPG) % CPR; }
-  // One chunk swizzle for a tile that is read both ways, so that it is stored once (the tiles that go from
-  // global memory straight into LDS): with a = (r / RPG) % CPR, the bits of a rotated so that its lowest
+  // One chunk swizzle for a tile that is read both ways, so that it is stored once: chunk c of row r sits
+  // at chunk position c ^ swz_both(r).  With a = (r / RPG) % CPR, the bits of a rotated so that its lowest
   // bits select the 64-byte column group.  Over any 16 consecutive rows the 16-byte slots of a chunk
   // column are all different (reads by rows), and rows 0-7 of a group spread evenly over the column
   // groups (transposing reads).

@@ -966,7 +966,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
           }
         }
         // The next tile's K is requested right after this tile's first operand reads, its V only after
-        // the first MFMA block: the four wavefronts then do not all queue at the load unit at once.
+        // the first MFMA block: the wavefronts then do not all queue at the load unit at once.
 
         const bool compute = active && (!p.causal || kpos <= wave_kvis_max);
         if (!compute && nx_valid > 0) {
