@@ -496,9 +496,12 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-template <int D, typename E, bool OUT32, int NW>
+template <int D, typename E, bool OUT32, int NW, bool EXTRAS>
 __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) {
   // OUT32: fp32 output (the fp32-input path; q/k/v are then fp16 staging copies)
+  // EXTRAS: the clocked walk, the split over key blocks and the log-sum-exp output are compiled in.  The
+  // plain call uses none of them, and its kernel is a tenth shorter without them (1-2 % faster: eight
+  // wavefronts in different parts of a long kernel share one instruction cache).
   // NW: wavefronts (wave slots) of a workgroup, 4 or 8.  Eight are used when the q heads of a GQA group
   // and the 32-row slices of a q block give an item more than four wave slots: one workgroup per CU then
   // stages every K/V tile once for all of them instead of two workgroups staging it each.
@@ -641,7 +644,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
   auto note_item = [&](int c_, int total_) {   // right after build(c_), from the staged records
     const int nkblk = __builtin_amdgcn_readlane((int)st_info, 6);
     const int seq = __builtin_amdgcn_readlane((int)st_info, 8);
-    w_part_of[c_] = p.walk != 0 && st_hk >= 0 && total_ >= 3 && total_ <= kListCap;
+    w_part_of[c_] = EXTRAS && p.walk != 0 && st_hk >= 0 && total_ >= 3 && total_ <= kListCap;
     w_clock_of[c_] = p.clock + (size_t)(st_hk < 0 ? 0 : st_hk) * p.nqb + seq;
     w_tiles_of[c_] = (nkblk * p.kbs + kTileKeys - 1) >> 6;
   };
@@ -889,7 +892,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
 
     if (wave == 0) {   // stay one item ahead: expand the staged item, stage the one after it
       build(c ^ 1);
-      if (p.walk) note_item(c ^ 1, hdr_word(c ^ 1, H_TOTAL));
+      if (EXTRAS && p.walk) note_item(c ^ 1, hdr_word(c ^ 1, H_TOTAL));
       stage();
       pending = claim();
     }
@@ -935,7 +938,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
         // The clock is dealt with on few tiles only (wavefront 0; any work it does alone on every tile
         // makes the other three wait at the next barrier): the item's first tile, every eighth, and
         // the last three.
-        if (p.walk && wave == 0 && ((t & (kWalkReportTiles - 1)) == 0 || chunk_base + t + 3 >= total)) {
+        if (EXTRAS && p.walk && wave == 0 && ((t & (kWalkReportTiles - 1)) == 0 || chunk_base + t + 3 >= total)) {
           report(c, kpos, chunk_base + t == 0, t + t0 >= n ? 1 : 0);
           if (chunk_base + t + 3 == total) peek_next(c ^ 1);
           if (chunk_base + t + 2 == total) next_start(c ^ 1);
@@ -1178,7 +1181,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
     if (active) {
       const float l_tot = half_sum(l_run);
       const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;   // 1 ulp; a full division is ten instructions
-      if (p.nparts > 1) {
+      if (EXTRAS && p.nparts > 1) {
         // split over key blocks: this part's normalised result and log-sum-exp, for the merge kernel
         if (l32 < nrows) {
           const int64_t rh = ((int64_t)cur_part * p.total_q + (row_begin + row0 + l32)) * p.nhead_q + hq;
@@ -1194,7 +1197,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
             }
         }
       } else {
-      if (p.lse != nullptr && g32 == 0 && l32 < nrows) {
+      if (EXTRAS && p.lse != nullptr && g32 == 0 && l32 < nrows) {
         // natural-log sum over the row's visible keys of exp(scale * q.k); m_run is the (possibly
         // lagging) reference maximum the row sum was accumulated under, which makes this exact
         const float lse = l_tot > 0.f ? (m_run * sm_c + __builtin_amdgcn_logf(l_tot)) * 0.69314718055994531f : -INFINITY;
@@ -1432,10 +1435,10 @@ int persistent_grid(const void *kernel, int lds_bytes, int threads) {
   return cus * per_cu;
 }
 
-template <int D, typename E, bool OUT32, int NW>
+template <int D, typename E, bool OUT32, int NW, bool EXTRAS>
 int launch_fwd_nw(const FwdParams &fp, long long items, hipStream_t stream) {
   constexpr int lds_bytes = 4 * kTileKeys * D * 2 + 2 * H_WORDS * 4 + 2 * kListCap * 4;
-  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E, OUT32, NW>);
+  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS>);
   // workgroups that fit the current device at once; the attribute and the occupancy are per device
   static thread_local int resident_of[kMaxDevices] = {};
   int dev = 0;
@@ -1449,17 +1452,19 @@ int launch_fwd_nw(const FwdParams &fp, long long items, hipStream_t stream) {
     if (resident <= 0) return fail(HBSA_ERR_UNSUPPORTED, "could not size the persistent grid");
   }
   const int grid = (int)(items < resident ? items : resident);
-  hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32, NW>), dim3(grid), dim3(NW * 64), lds_bytes, stream, fp);
+  hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS>), dim3(grid), dim3(NW * 64), lds_bytes, stream, fp);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail((int)e, "hbsa_fwd_kernel launch: %s", hipGetErrorString(e));
   return 0;
 }
 template <int D, typename E, bool OUT32>
 int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
+  const bool extras = fp.walk != 0 || fp.nparts > 1 || fp.lse != nullptr;
   if constexpr (D >= 64) {
-    if (fp.nw == 8) return launch_fwd_nw<D, E, OUT32, 8>(fp, items, stream);
+    if (fp.nw == 8)
+      return extras ? launch_fwd_nw<D, E, OUT32, 8, true>(fp, items, stream) : launch_fwd_nw<D, E, OUT32, 8, false>(fp, items, stream);
   }
-  return launch_fwd_nw<D, E, OUT32, 4>(fp, items, stream);
+  return extras ? launch_fwd_nw<D, E, OUT32, 4, true>(fp, items, stream) : launch_fwd_nw<D, E, OUT32, 4, false>(fp, items, stream);
 }
 
 
