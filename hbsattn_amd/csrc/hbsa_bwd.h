@@ -41,6 +41,7 @@ struct BwdParams {
   const int32_t *cu_k, *cu_num_q_block, *cu_num_k_block;
   int64_t q_s, q_h, k_s, k_h, v_s, v_h, o_s, o_h, do_s, do_h, dq_s, dq_h, dk_s, dk_h, dv_s, dv_h;   // bytes
   int32_t nqb, nkb, xcd_heads, batch, ratio, nhead_q, qbs, kbs, wpr, causal;   // xcd_heads: see the dK/dV kernels
+  int32_t total_k;
   int32_t wps, nsub;     // q side: wave slots per q head and workgroups per (kv head, q block), as in the forward
   int32_t nsub_k;        // k side: workgroups per (kv head, k block) = ceil(k_block_size / 128)
   float c;               // softmax_scale * log2(e), signed
@@ -135,6 +136,32 @@ __device__ __forceinline__ void bwd_store_rows(char *row_ptr, const f32x16 *acc,
     }
 }
 
+// The dK/dV kernels' check of the sequence b their k block belongs to.  A sequence the pre-pass found not to
+// fit the tensors (flagged q block records, no bit rows) takes no part: its keys get zero gradients where they
+// lie inside dk and dv, and the workgroup is done.
+template <int D>
+__device__ __forceinline__ bool bwd_sequence_skipped(const BwdParams &p, int b, int kb, int sub, int hk) {
+  const int first_qb = p.cu_num_q_block[b];
+  if (first_qb < 0 || first_qb >= p.nqb) return true;
+  if (first_qb >= p.cu_num_q_block[b + 1] || p.info[first_qb].flags == 0) return false;
+  const int64_t k0 = p.cu_k[b], k1 = p.cu_k[b + 1];
+  const int kbl = kb - p.cu_num_k_block[b];
+  if (k0 < 0 || k1 <= k0 || kbl < 0) return true;
+  const int64_t first = k0 + (int64_t)kbl * p.kbs + (int64_t)sub * 4 * kWaveRows;
+  int64_t stop = k0 + (int64_t)(kbl + 1) * p.kbs;
+  stop = stop < k1 ? stop : k1;
+  stop = stop < first + 4 * kWaveRows ? stop : first + 4 * kWaveRows;
+  stop = stop < p.total_k ? stop : (int64_t)p.total_k;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  for (int64_t i = threadIdx.x; i < (stop - first) * (D / 8); i += blockDim.x) {
+    const int64_t row = first + i / (D / 8);
+    const int c = (int)(i % (D / 8));
+    *(u32x4 *)(p.dk + row * p.dk_s + (int64_t)hk * p.dk_h + c * 16) = zero;
+    *(u32x4 *)(p.dv + row * p.dv_s + (int64_t)hk * p.dv_h + c * 16) = zero;
+  }
+  return true;
+}
+
 // ---- dQ ----------------------------------------------------------------------------------------------
 template <int D, typename E>
 __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
@@ -157,7 +184,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   const int qb_rev = bx / p.nsub, sub = bx - qb_rev * p.nsub;
   const int qb = p.nqb - 1 - qb_rev;
   const QBlockInfo inf = p.info[qb];
-  if (inf.rows <= 0) return;   // a q block of a sequence the pre-pass skipped (boundaries outside the tensors)
+  if (inf.rows <= 0) return;   // a q block with no row inside the tensors (its sequence did not fit them)
 
   const int slot = sub * 4 + wave;
   const int head_in_group = slot / p.wps;
@@ -314,10 +341,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dkv_kernel(BwdParams p) 
 
   int b = 0;   // the sequence the k block belongs to
   while (b + 1 < p.batch && p.cu_num_k_block[b + 1] <= kb) ++b;
-  {   // a sequence the pre-pass skipped (boundaries outside the tensors) has empty q block records: nothing to do
-    const int first_qb = p.cu_num_q_block[b];
-    if (first_qb < 0 || first_qb >= p.nqb || (first_qb < p.cu_num_q_block[b + 1] && p.info[first_qb].rows <= 0)) return;
-  }
+  if (bwd_sequence_skipped<D>(p, b, kb, sub, hk)) return;
   const int kbl = kb - p.cu_num_k_block[b];          // in-sequence index of the k block
   const int k0 = p.cu_k[b], klen = p.cu_k[b + 1] - k0;
   const int krows = min(p.kbs, klen - kbl * p.kbs);  // keys in the block
@@ -542,10 +566,7 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
 
   int b = 0;   // the sequence the k block belongs to
   while (b + 1 < p.batch && p.cu_num_k_block[b + 1] <= kb) ++b;
-  {   // a sequence the pre-pass skipped (boundaries outside the tensors) has empty q block records: nothing to do
-    const int first_qb = p.cu_num_q_block[b];
-    if (first_qb < 0 || first_qb >= p.nqb || (first_qb < p.cu_num_q_block[b + 1] && p.info[first_qb].rows <= 0)) return;
-  }
+  if (bwd_sequence_skipped<D>(p, b, kb, sub, hk)) return;
   const int kbl = kb - p.cu_num_k_block[b];
   const int k0 = p.cu_k[b], klen = p.cu_k[b + 1] - k0;
   const int krows = min(p.kbs, klen - kbl * p.kbs);

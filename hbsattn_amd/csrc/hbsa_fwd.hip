@@ -71,8 +71,10 @@ struct QBlockInfo {
   int32_t shift;       // k_len - q_len: bottom-right causal alignment
   int32_t nkblk;       // k blocks in the sequence
   int32_t kmax;        // exclusive in-sequence bound of keys any row of the block may see
-  int32_t seq;         // index of the sequence in the packed batch
-  int32_t pad[3];
+  int32_t seq;         // first q block of the block's sequence: identifies the sequence by a number below num_q_block
+                       // (the batch index can exceed it when the batch holds sequences without queries)
+  int32_t flags;       // 1: the block's sequence did not fit the tensors; it has no keys (and perhaps no rows)
+  int32_t pad[2];
 };
 static_assert(sizeof(QBlockInfo) == 48, "QBlockInfo is read as twelve 32-bit words");
 
@@ -128,7 +130,7 @@ struct FwdParams {
   // one (kv head, sequence) keep near each other in key space through a shared clock, so that they find
   // each other's K/V blocks in the L2; the summation order, and with it the last bits of the result,
   // then depend on timing.  walk == 0: every item walks its blocks in ascending order (deterministic).
-  unsigned long long *clock;   // [nhead_k, num_q_block]: clock of (kv head, sequence index)
+  unsigned long long *clock;   // [nhead_k, num_q_block]: clock of (kv head, first q block of the sequence)
   int32_t walk;
   float *lse;             // optional [total_q, nhead_q] log-sum-exp output (nullptr: none)
   int64_t lse_s, lse_h;   // its strides in elements
@@ -142,6 +144,56 @@ struct FwdParams {
   int32_t total_q, nhead_q;
 };
 
+// Boundaries of one sequence of the packed batch, as read from the caller's device arrays.
+struct SeqBounds {
+  int32_t q0, q1;     // cu_q_seqlens[b], [b + 1]
+  int32_t k0, k1;     // cu_k_seqlens[b], [b + 1]
+  int32_t kb0, kb1;   // cu_num_k_block[b], [b + 1]
+  int32_t qb0;        // cu_num_q_block[b]
+};
+
+// Geometry record of q block g.  The sequence boundaries are device data the host cannot check, so they
+// are checked here against the token counts of q and k/v and the block counts.  A sequence that does
+// not fit (a wrong cu_seqlens, q/k/v shorter than it says, inconsistent block metadata) gets no keys:
+// nothing of k, v or the mask is read for it, and those of its query rows that lie inside q and out are
+// written as zeros, like any row that sees no key (flags = 1 marks such a block).  When not even the
+// query side makes sense (have == false: the block's sequence index is outside the batch) the block
+// has no rows and nothing is written for it.  kb0: first global k block of the sequence.
+__host__ __device__ inline QBlockInfo q_block_geometry(int g, bool have, SeqBounds s, int qbs, int kbs, int causal,
+                                                      int nkb_total, int total_q, int total_k, int &kb0) {
+  const int qlen = s.q1 - s.q0, klen_in = s.k1 - s.k0, nkb_in = s.kb1 - s.kb0;
+  const int q_pos = (g - s.qb0) * qbs;
+  const bool q_ok = have && s.q0 >= 0 && qlen > 0 && s.qb0 >= 0 && g >= s.qb0 && q_pos >= 0 && q_pos < qlen &&
+                    (int64_t)s.q0 + q_pos < total_q;
+  const bool ok = q_ok && (int64_t)s.q0 + qlen <= total_q && s.k0 >= 0 && klen_in >= 0 && (int64_t)s.k0 + klen_in <= total_k &&
+                  s.kb0 >= 0 && nkb_in >= 0 && (int64_t)s.kb0 + nkb_in <= nkb_total && (int64_t)nkb_in * kbs >= klen_in;
+  QBlockInfo r;
+  r.row_begin = q_ok ? s.q0 + q_pos : 0;
+  int rows = 0;
+  if (q_ok) {
+    rows = qlen - q_pos < qbs ? qlen - q_pos : qbs;
+    if (rows > total_q - r.row_begin) rows = total_q - r.row_begin;
+  }
+  r.rows = rows;
+  r.key_begin = ok ? s.k0 : 0;
+  r.klen = ok ? klen_in : 0;
+  r.q_pos = q_ok ? q_pos : 0;
+  r.shift = ok ? klen_in - qlen : 0;
+  r.nkblk = ok ? nkb_in : 0;
+  int kmax = 0;
+  if (ok) {
+    kmax = klen_in;
+    if (causal && q_pos + rows + r.shift < kmax) kmax = q_pos + rows + r.shift;
+    if (kmax < 0) kmax = 0;
+  }
+  r.kmax = kmax;
+  r.seq = q_ok ? s.qb0 : 0;
+  r.flags = ok ? 0 : 1;
+  r.pad[0] = r.pad[1] = 0;
+  kb0 = ok ? s.kb0 : 0;
+  return r;
+}
+
 // --------------------------------------------------------------------------------------
 // Pre-pass: one wavefront per (kv head, q block).
 // --------------------------------------------------------------------------------------
@@ -153,33 +205,19 @@ __global__ __launch_bounds__(kThreads) void hbsa_prep_kernel(PrepParams p) {
   if (g >= p.nqb) return;
   const int hk = blockIdx.y;
   const int b = p.q_block_to_batch[g];
-  // A sequence whose boundaries do not fit the tensors and the block counts (a wrong cu_seqlens, q/k/v
-  // shorter than it says) is skipped as a whole: its q blocks get empty records and bit rows, which
-  // every kernel that reads them treats as "nothing to do", so nothing outside the tensors is touched.
-  bool ok = b >= 0 && b < p.batch;
-  int q0 = 0, qlen = 0, k0 = 0, klen = 0, kb0 = 0, nkb = 0, q_pos = 0;
-  if (ok) {
-    q0 = p.cu_q[b]; qlen = p.cu_q[b + 1] - q0;
-    k0 = p.cu_k[b]; klen = p.cu_k[b + 1] - k0;
-    kb0 = p.cu_num_k_block[b]; nkb = p.cu_num_k_block[b + 1] - kb0;
-    const int qb0 = p.cu_num_q_block[b];
-    q_pos = (g - qb0) * p.qbs;
-    ok = q0 >= 0 && qlen > 0 && (int64_t)q0 + qlen <= p.total_q && k0 >= 0 && klen >= 0 && (int64_t)k0 + klen <= p.total_k &&
-         kb0 >= 0 && nkb >= 0 && (int64_t)kb0 + nkb <= p.nkb && (int64_t)nkb * p.kbs >= klen && g >= qb0 && q_pos < qlen;
+  SeqBounds sb = {0, 0, 0, 0, 0, 0, 0};
+  const bool have = b >= 0 && b < p.batch;
+  if (have) {
+    sb.q0 = p.cu_q[b]; sb.q1 = p.cu_q[b + 1];
+    sb.k0 = p.cu_k[b]; sb.k1 = p.cu_k[b + 1];
+    sb.kb0 = p.cu_num_k_block[b]; sb.kb1 = p.cu_num_k_block[b + 1];
+    sb.qb0 = p.cu_num_q_block[b];
   }
-  if (!ok) { q0 = qlen = k0 = klen = kb0 = nkb = q_pos = 0; }
-  const int rows = ok ? min(p.qbs, qlen - q_pos) : 0;
-  const int shift = klen - qlen;
-  int kmax = p.causal ? min(klen, q_pos + rows + shift) : klen;
-  if (kmax < 0 || !ok) kmax = 0;
-  const int nvis = min(nkb, (kmax + p.kbs - 1) / p.kbs);
-  if (hk == 0 && lane == 0) {
-    QBlockInfo r;
-    r.row_begin = q0 + q_pos; r.rows = rows; r.key_begin = k0; r.klen = klen;
-    r.q_pos = q_pos; r.shift = shift; r.nkblk = nkb; r.kmax = kmax;
-    r.seq = ok ? b : 0; r.pad[0] = r.pad[1] = r.pad[2] = 0;
-    p.info[g] = r;
-  }
+  int kb0;
+  const QBlockInfo r = q_block_geometry(g, have, sb, p.qbs, p.kbs, p.causal, p.nkb, p.total_q, p.total_k, kb0);
+  const int nkb = r.nkblk;
+  const int nvis = min(nkb, (r.kmax + p.kbs - 1) / p.kbs);
+  if (hk == 0 && lane == 0) p.info[g] = r;
   if (lane == 0) p.clock[(size_t)hk * p.nqb + g] = 0ull;   // the walk clocks start at zero (and every launch leaves them so)
   uint32_t *row = p.bits + ((size_t)hk * p.nqb + g) * p.wpr;
   const uint8_t *m = p.mask + hk * p.ms_h + g * p.ms_q + kb0 * p.ms_k;
@@ -1354,12 +1392,13 @@ inline size_t bits_offset(int nhead_k, int num_q_block) {
   return clock_offset(num_q_block) + align_up((size_t)nhead_k * num_q_block * sizeof(unsigned long long), 256);
 }
 
-// Deterministic mode: every item walks its tiles in ascending order, so results are bitwise
-// reproducible; otherwise very large problems use the clocked walk (results then vary in their last
-// bits from run to run).  Initial value from the environment variable HBSATTN_AMD_DETERMINISTIC.
+// Deterministic mode (the default, like the reference's ascending scan): every item walks its tiles in
+// ascending order, so results are bitwise reproducible.  With it switched off (hbsa_set_deterministic(0) or
+// the environment variable HBSATTN_AMD_DETERMINISTIC=0) very large problems use the clocked walk, and
+// results then vary in their last bits from run to run.
 int g_deterministic = [] {
   const char *e = std::getenv("HBSATTN_AMD_DETERMINISTIC");
-  return e != nullptr && e[0] != 0 && e[0] != '0' ? 1 : 0;
+  return e != nullptr && e[0] == '0' && e[1] == 0 ? 0 : 1;
 }();
 // K + V bytes of one kv head from which the clocked walk is used.  Measured on MI355X: at 64K-token
 // sequences with 30 % of the blocks kept the walk takes a seventh off the HBM traffic and 5 % off the
@@ -2072,7 +2111,7 @@ int hbsa_bwd(const void *q, const void *k, const void *v, const void *out, const
   bp.do_s = strides[8] * es; bp.do_h = strides[9] * es;
   bp.dq_s = strides[10] * es; bp.dq_h = strides[11] * es; bp.dk_s = strides[12] * es; bp.dk_h = strides[13] * es;
   bp.dv_s = strides[14] * es; bp.dv_h = strides[15] * es;
-  bp.nqb = num_q_block; bp.nkb = num_k_block; bp.batch = batch;
+  bp.nqb = num_q_block; bp.nkb = num_k_block; bp.batch = batch; bp.total_k = total_k;
   bp.ratio = nhead_q / nhead_k; bp.nhead_q = nhead_q; bp.qbs = q_block_size;
   bp.kbs = k_block_size;
   bp.wpr = words_per_row(num_k_block); bp.causal = causal ? 1 : 0;

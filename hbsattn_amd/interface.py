@@ -42,11 +42,12 @@ def set_fp32_mode(mode: str) -> str:
 
 
 def set_deterministic(on: bool) -> bool:
-    """Deterministic mode of the library (``hbsa_set_deterministic``): with it on every query block walks
-    its key tiles in ascending order and results are bitwise reproducible at every size; with it off
-    (the default unless HBSATTN_AMD_DETERMINISTIC is set) very large problems order the walk by a clock
-    shared between workgroups, which saves HBM traffic and lets the last bits of the result depend on
-    timing.  Returns the previous setting."""
+    """Deterministic mode of the library (``hbsa_set_deterministic``), on by default: every query block
+    walks its key tiles in ascending order and results are bitwise reproducible at every size, like the
+    reference's kernels.  Switched off (here, or with HBSATTN_AMD_DETERMINISTIC=0 in the environment when
+    the library is loaded), very large problems order the walk by a clock shared between workgroups,
+    which saves HBM traffic and lets the last bits of the result depend on timing.  Returns the previous
+    setting."""
     return bool(_lib.load().hbsa_set_deterministic(1 if on else 0))
 
 
@@ -96,6 +97,14 @@ class PreparedMask:
         self.q_block_size = q_block_size
         self.k_block_size = k_block_size
         self.causal = bool(causal)
+
+    def skipped_q_blocks(self) -> int:
+        """Number of q blocks whose sequence did not fit the tensors it was prepared for (boundaries beyond
+        the token counts of q or k/v, inconsistent block metadata).  Such sequences get no keys: their
+        output rows and gradients are zeros.  Reads device memory (synchronises): for diagnostics, not
+        for the hot path."""
+        records = self.workspace[: self.num_q_block * 48].view(torch.int32).view(self.num_q_block, 12)
+        return int(records[:, 9].ne(0).sum())
 
 
 def _check_on_device(dev, **tensors):
@@ -327,12 +336,15 @@ def clear_prepared_cache() -> None:
 
 def _cached_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, num_q_block,
                     q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, run_shape) -> PreparedMask:
-    tensors = (block_mask, cu_q_seqlens, cu_k_seqlens)
+    # everything the pre-pass reads or bakes in: the mask, the boundaries, the block metadata, and the
+    # token counts the boundaries were checked against
+    tensors = (block_mask, cu_q_seqlens, cu_k_seqlens, q_block_to_batch, cu_num_q_block, cu_num_k_block)
     key = None
     if _prepared_cache_size > 0 and all(isinstance(t, torch.Tensor) for t in tensors) and block_mask.is_cuda:
         try:
             key = tuple((id(t), t._version, t.data_ptr(), tuple(t.shape), tuple(t.stride())) for t in tensors) + (
                 int(q_block_size), int(k_block_size), bool(causal), int(num_q_block), int(num_k_block),
+                None if run_shape is None else (int(run_shape[1]), int(run_shape[2])),
                 block_mask.device.index, torch.cuda.current_stream(block_mask.device).cuda_stream)
         except RuntimeError:   # tensors without a version counter (inference mode): no reuse
             key = None

@@ -42,8 +42,8 @@ def test_workspace_bytes_is_host_only_and_monotone():
     c = lib.hbsa_fwd_workspace_bytes(32, 4096, 4096)
     assert 0 < a < b < c
     assert a % 256 == 0 and b % 256 == 0
-    # one bit per k block per (kv head, q block) plus a 32-byte record per q block
-    assert b >= 32 * 2048 * (2048 // 8) + 2048 * 32
+    # one bit per k block per (kv head, q block) plus a 48-byte record per q block
+    assert b >= 32 * 2048 * (2048 // 8) + 2048 * 48
     assert c < 80 * 2 ** 20
 
 

@@ -484,8 +484,9 @@ def test_clocked_walk_matches_the_oracle_and_leaves_its_clocks_at_zero(causal, k
     ref = oracle_for(w)
     straight = _run(w)                                      # ascending walk (the problem is far below the threshold)
     previous = lib.hbsa_set_walk_min_bytes(0)
+    was_deterministic = lib.hbsa_set_deterministic(0)       # the clocked walk is opt-in
     try:
-        assert not lib.hbsa_set_deterministic(0)
+        assert was_deterministic == 1, "the ascending, reproducible walk is the library's default"
         prepared = hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, qbs, kbs, causal, w.q_meta[0], w.q_meta[2],
                                 w.q_meta[3], w.k_meta[0], w.k_meta[3])
         nqb, nhk = w.q_meta[0], w.k.shape[1]
@@ -501,15 +502,51 @@ def test_clocked_walk_matches_the_oracle_and_leaves_its_clocks_at_zero(causal, k
         lib.hbsa_set_deterministic(1)
         assert torch.equal(hbsa_run(w.q, w.k, w.v, prepared, None), straight)
     finally:
-        lib.hbsa_set_deterministic(0)
+        lib.hbsa_set_deterministic(was_deterministic)
+        lib.hbsa_set_walk_min_bytes(previous)
+
+
+def test_clocked_walk_with_sequences_that_have_no_queries():
+    """A batch may hold more sequences than q blocks (sequences without queries).  The walk clocks are
+    one word per (kv head, q block); a sequence is identified by its first q block, which stays inside
+    that array whatever the batch index is."""
+    from hbsattn_amd import _lib
+    from hbsattn_amd.interface import hbsa_prepare, hbsa_run
+    lib = _lib.load()
+    w = make_problem(seed=95, q_lens=[256, 0, 0, 0, 0, 384], k_lens=[512, 128, 64, 256, 128, 640], hq=4, hk=4, d=128, qbs=128,
+                     kbs=64, keep=0.5, diag=True, causal=True, scale=None)
+    assert len(w.cu_q) - 1 > w.q_meta[0]                     # more sequences than q blocks
+    ref = oracle_for(w)
+    straight = _run(w)
+    assert_close_to_oracle(straight, ref, "ascending walk")
+    previous = lib.hbsa_set_walk_min_bytes(0)
+    was_deterministic = lib.hbsa_set_deterministic(0)
+    try:
+        prepared = hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, 128, 64, True, w.q_meta[0], w.q_meta[2],
+                                w.q_meta[3], w.k_meta[0], w.k_meta[3])
+        nqb, nhk = w.q_meta[0], w.k.shape[1]
+        clock_at = (nqb * 48 + 255) // 256 * 256 + 256
+        bits_at = clock_at + (8 * nhk * nqb + 255) // 256 * 256
+        bits_end = bits_at + nhk * nqb * 2 * ((w.k_meta[0] + 63) // 64) * 4
+        bits_before = prepared.workspace[bits_at:bits_end].clone()
+        for launch in range(2):
+            out = hbsa_run(w.q, w.k, w.v, prepared, None)
+            torch.cuda.synchronize()
+            assert_close_to_oracle(out, ref, f"clocked walk, launch {launch}")
+            assert int(prepared.workspace[clock_at:clock_at + 8 * nhk * nqb].view(torch.int64).abs().max()) == 0
+            assert torch.equal(prepared.workspace[bits_at:bits_end], bits_before), "a clock update landed in the bit rows"
+    finally:
+        lib.hbsa_set_deterministic(was_deterministic)
         lib.hbsa_set_walk_min_bytes(previous)
 
 
 def test_a_sequence_that_does_not_fit_the_tensors_is_skipped_not_read_out_of_bounds():
-    """cu_seqlens that promise more tokens than q (or k, v) hold: the pre-pass checks every sequence
-    against the tensors' token counts and leaves out the one that does not fit, so the others come out
-    exactly as in the full problem and nothing beyond the tensors is touched.  (The short tensors are
-    views of the full ones, so the check is what keeps the kernels inside them, not luck.)"""
+    """cu_seqlens that promise more tokens than q (or k, v) hold: every sequence is checked on the device
+    against the tensors' token counts and the one that does not fit gets no keys, so the others come out
+    exactly as in the full problem, nothing beyond the tensors is touched, and those of its query rows that
+    exist are defined (zeros, like any row without keys).  (The short tensors are views of the full ones,
+    so the check is what keeps the kernels inside them, not luck.)"""
+    from hbsattn_amd.interface import hbsa_prepare
     w = make_problem(seed=94, q_lens=[300, 500, 200], k_lens=[300, 500, 260], hq=4, hk=2, d=64, qbs=64, kbs=64, keep=0.5,
                      diag=True, causal=True, scale=None)
     full = _run(w)
@@ -518,12 +555,21 @@ def test_a_sequence_that_does_not_fit_the_tensors_is_skipped_not_read_out_of_bou
     out = HBSAttention(*args)
     torch.cuda.synchronize()
     assert out.shape[0] == 900 and torch.equal(out[:800], full[:800])
+    assert int(out[800:].ne(0).sum()) == 0, "rows of the sequence that does not fit are zeros"
     args = list(w.args())
     args[1], args[2] = w.k[:1000], w.v[:1000]  # the third sequence's keys would be rows 800 .. 1059
     out = HBSAttention(*args)
     torch.cuda.synchronize()
     assert torch.equal(out[:800], full[:800])
-    # and the backward: gradients of the sequences that fit are those of the full problem
+    assert int(out[800:].ne(0).sum()) == 0
+    # the skip can be observed (off the hot path: it reads device memory)
+    meta = (w.q_meta[0], w.q_meta[2], w.q_meta[3], w.k_meta[0], w.k_meta[3])
+    fits = hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, 64, 64, True, *meta,
+                        run_shape=(w.q.dtype, 1000, 1060, 4, 64))
+    short = hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, 64, 64, True, *meta,
+                         run_shape=(w.q.dtype, 900, 1060, 4, 64))
+    assert fits.skipped_q_blocks() == 0 and short.skipped_q_blocks() == 4   # the 200-row sequence has four 64-row blocks
+    # and the backward: gradients of the sequences that fit are those of the full problem, the rest zeros
     q, k, v = (t.detach().clone().requires_grad_(True) for t in (w.q, w.k, w.v))
     args = list(w.args())
     args[:3] = [q, k, v]
@@ -535,6 +581,7 @@ def test_a_sequence_that_does_not_fit_the_tensors_is_skipped_not_read_out_of_bou
     torch.cuda.synchronize()
     assert torch.equal(q2.grad[:800], q.grad[:800])
     assert torch.equal(k2.grad[:800], k.grad[:800]) and torch.equal(v2.grad[:800], v.grad[:800])
+    assert int(q2.grad[800:].ne(0).sum()) == 0 and int(k2.grad[800:].ne(0).sum()) == 0 and int(v2.grad[800:].ne(0).sum()) == 0
 
 
 def test_prepared_masks_are_reused_only_for_unchanged_tensors():
@@ -558,9 +605,17 @@ def test_prepared_masks_are_reused_only_for_unchanged_tensors():
             assert_close_to_oracle(_run(w), oracle_for(w), "other stream")
         torch.cuda.synchronize()
         assert len(calls) == 3
+        # shorter q on the same mask and boundaries: the prepared bounds check belonged to the longer tensors,
+        # so the call prepares again (and the sequence that no longer fits is left out, not read out of bounds)
+        args = list(w.args())
+        args[0] = w.q[:1000]
+        short = HBSAttention(*args)
+        torch.cuda.synchronize()
+        assert len(calls) == 4 and torch.equal(short[:700], _run(w)[:700]) and int(short[700:].ne(0).sum()) == 0
+        assert len(calls) == 4                                   # ... and the full-length entry is still there
         set_prepared_cache_size(0)                               # switched off: every call prepares
         _run(w), _run(w)
-        assert len(calls) == 5
+        assert len(calls) == 6
     finally:
         interface.hbsa_prepare = real
         set_prepared_cache_size(previous)
