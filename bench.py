@@ -8,7 +8,8 @@ after it and reported under ``other_shapes``.  Every workload runs the library's
 ascending walk except C4, whose headline figures use the opt-in clocked walk (``walk`` says which; C4's
 ascending-walk kernel time is reported beside it).
 
-A step is one ``HBSAttention`` call (pre-pass + attention kernel, block metadata
+A step is one ``HBSAttention`` call (one launch: the attention kernel, whose scheduler reads the mask
+itself; pre-pass + attention kernel where that form does not apply; block metadata
 pre-computed and passed in as the reference's sweep does, reference
 test/test_speedup.py:101-102,152) on a synthetic problem already resident in HBM.  The
 timed region is ``synchronize -> K calls -> synchronize`` (reference hbsattn/benchmark.py:72-81
@@ -145,9 +146,22 @@ def measure(name, steps, warmup):
     return w, res
 
 
+def settle(fn, seconds=0.25):
+    """Set-up before any measurement of a workload: calls until `seconds` of wall time have passed, so that the
+    device has left its idle clocks, the allocator holds the output buffer and every page of the tensors has been
+    touched.  (Measured without it, the first 20 ms after a workload is built run a tenth slower, which is what a
+    short workload's whole measurement takes.)  The W warm-up steps and the K timed steps come after it."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
+
+
 def _measure(w, work, name, steps, warmup, HBSAttention, hbsa_prepare, hbsa_run):
     args = w.args()
     step = lambda: HBSAttention(*args)
+    settle(step)
     ms = time_steps(step, steps, warmup)
     per_call = time_per_call_sync(step, steps)
     # the same with the prepared mask of the first call reused by the following ones (opt-in mode of the
@@ -159,15 +173,24 @@ def _measure(w, work, name, steps, warmup, HBSAttention, hbsa_prepare, hbsa_run)
     clear_prepared_cache()
     prepared = hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, w.q_block_size, w.k_block_size, w.causal,
                             w.q_meta[0], w.q_meta[2], w.q_meta[3], w.k_meta[0], w.k_meta[3])
-    kernel_ms = time_kernel_events(lambda: hbsa_run(w.q, w.k, w.v, prepared, w.softmax_scale), steps)
+    prepared_kernel_ms = time_kernel_events(lambda: hbsa_run(w.q, w.k, w.v, prepared, w.softmax_scale), steps)
     prep_ms = time_kernel_events(
         lambda: hbsa_prepare(w.cu_q_seqlens, w.cu_k_seqlens, w.block_mask, w.q_block_size, w.k_block_size, w.causal,
                              w.q_meta[0], w.q_meta[2], w.q_meta[3], w.k_meta[0], w.k_meta[3]), steps)
+    # the launches a step makes: 1 = the attention kernel alone, its scheduler reading the mask itself (then the
+    # events around a whole call bracket exactly that kernel), 2 = pre-pass + attention kernel on a workspace
+    from hbsattn_amd import _lib
+    launches = _lib.load().hbsa_fwd_launches(_lib.DTYPE_BF16, len(w.cu_q) - 1, w.k.shape[0], w.q.shape[1], w.k.shape[1],
+                                             w.q.shape[2], w.q_meta[0], w.k_meta[0], w.q_block_size, w.k_block_size,
+                                             w.block_mask.stride(2), torch.cuda.current_stream().cuda_stream)
+    kernel_ms = time_kernel_events(step, steps) if launches == 1 else prepared_kernel_ms
     res = {
         "ms_per_step": ms,
         "per_call_sync_ms": per_call,
         "ms_per_step_mask_reused": ms_reused,
+        "launches_per_step": launches,
         "attention_kernel_ms": kernel_ms,
+        "attention_kernel_ms_on_prepared_mask": prepared_kernel_ms,
         "prepass_ms": prep_ms,
         "tflops": work["flops"] / ms / 1e9,
         "tflops_exact_elements": work["flops_exact"] / ms / 1e9,
@@ -308,7 +331,8 @@ def main():
                    "block metadata precomputed; one HBSAttention call per step"},
         "roofline": res["roofline"],
         "walk": res["walk"],
-        "detail": {k: res[k] for k in ("per_call_sync_ms", "ms_per_step_mask_reused", "attention_kernel_ms", "prepass_ms", "tflops_exact_elements",
+        "detail": {k: res[k] for k in ("launches_per_step", "per_call_sync_ms", "ms_per_step_mask_reused", "attention_kernel_ms",
+                                       "attention_kernel_ms_on_prepared_mask", "prepass_ms", "tflops_exact_elements",
                                        "flops", "bytes", "visited_pairs")},
     }
     if a.workload == "T":
@@ -328,7 +352,9 @@ def main():
             torch.cuda.empty_cache()
             line["other_shapes"][name] = {"workload": DESCRIPTIONS[name], "ms_per_step": t["ms_per_step"],
                                           "ms_per_step_mask_reused": t["ms_per_step_mask_reused"],
+                                          "launches_per_step": t["launches_per_step"],
                                           "tflops": t["tflops"], "attention_kernel_ms": t["attention_kernel_ms"],
+                                          "attention_kernel_ms_on_prepared_mask": t["attention_kernel_ms_on_prepared_mask"],
                                           "prepass_ms": t["prepass_ms"], "walk": t["walk"], "roofline": t["roofline"]}
             if "attention_kernel_ms_ascending_walk" in t:
                 line["other_shapes"][name]["attention_kernel_ms_ascending_walk"] = t["attention_kernel_ms_ascending_walk"]

@@ -6,12 +6,13 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhbsattn_amd.so")
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 DTYPE_BF16 = 0
 DTYPE_F16 = 1
 DTYPE_F32 = 2
 DTYPE_F32_STAGED16 = 3
+ERR_WORKSPACE_TOO_SMALL = -3
 STATIC_SCRATCH_BYTES = 32 << 20   # HBSA_STATIC_SCRATCH_BYTES of include/hbsattn_amd.h
 
 _lib = None
@@ -39,6 +40,10 @@ def load() -> ctypes.CDLL:
     lib.hbsa_last_error.argtypes = []
     lib.hbsa_set_deterministic.restype = ctypes.c_int
     lib.hbsa_set_deterministic.argtypes = [ctypes.c_int]
+    lib.hbsa_fwd_launches.restype = ctypes.c_int
+    lib.hbsa_fwd_launches.argtypes = [ctypes.c_int32] * 10 + [ctypes.c_int64, ctypes.c_void_p]
+    lib.hbsa_set_onepass.restype = ctypes.c_int
+    lib.hbsa_set_onepass.argtypes = [ctypes.c_int]
     lib.hbsa_set_walk_min_bytes.restype = ctypes.c_longlong
     lib.hbsa_set_walk_min_bytes.argtypes = [ctypes.c_longlong]
     lib.hbsa_fwd_workspace_bytes.restype = ctypes.c_size_t
@@ -50,6 +55,12 @@ def load() -> ctypes.CDLL:
     lib.hbsa_fwd.argtypes = ([vp] * 11 + [ctypes.c_size_t] + [ctypes.c_int32] * 12 + [ctypes.c_float]
                              + [ctypes.POINTER(ctypes.c_int64), vp])
     i64p = ctypes.POINTER(ctypes.c_int64)
+    # hbsa_fwd_v through a handle that keeps the interpreter lock during the call: its argument arrays are
+    # kept per shape and refilled per call, so no other Python thread may refill them while the library reads them
+    locked = ctypes.PyDLL(LIB_PATH)
+    lib.hbsa_fwd_v_locked = locked.hbsa_fwd_v
+    lib.hbsa_fwd_v_locked.restype = ctypes.c_int
+    lib.hbsa_fwd_v_locked.argtypes = [vp, ctypes.c_size_t, vp, ctypes.c_float, vp, vp]
     lib.hbsa_fwd_static.restype = ctypes.c_int
     lib.hbsa_fwd_static.argtypes = [vp] * 10 + [ctypes.c_int32] * 12 + [ctypes.c_float, i64p, vp]
     lib.hbsa_fwd_prepare.restype = ctypes.c_int

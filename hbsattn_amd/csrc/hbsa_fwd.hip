@@ -125,6 +125,7 @@ struct FwdParams {
   int32_t f32;    // fp32 inputs staged as fp16: the softmax constants come from the launch record, where
                   // the setup kernel derived them from the tensors' maxima
   int32_t nhead_k;
+  int32_t one_each;   // the grid has one workgroup per work item: workgroup i takes item i, the queues are not used
   struct Sched *sched;
   // Walk order of the kept k blocks (see the kernel's comment).  walk != 0: the workgroups that work on
   // one (kv head, sequence) keep near each other in key space through a shared clock, so that they find
@@ -142,6 +143,12 @@ struct FwdParams {
   float *part_out;        // [nparts, total_q, nhead_q, D]
   float *part_lse;        // [nparts, total_q, nhead_q]
   int32_t total_q, nhead_q;
+  // One-launch form (the kernel instantiated with FUSED): no pre-pass has run, `info` and `bits` are unused,
+  // and the scheduler derives every item's geometry and bit row itself from the caller's arrays.
+  const int32_t *cu_q, *cu_k, *cu_nqb, *cu_nkb;   // int32[batch + 1] each
+  const uint8_t *mask;                            // block_mask bytes, innermost (k block) stride 1
+  int64_t ms_h, ms_q;                             // its head and q block strides
+  int32_t batch, nkb_total, total_k, qbs;
 };
 
 // Boundaries of one sequence of the packed batch, as read from the caller's device arrays.
@@ -392,6 +399,11 @@ __global__ __launch_bounds__(256) void hbsa_f32_stage_kernel(F32Tensor t, const 
 }
 
 constexpr int kListCap = 1024;   // tile entries per list; longer items are expanded in chunks
+// One-launch form: sequences whose boundaries the scheduler keeps in LDS (batch + 1 entries of four arrays),
+// and bytes of its staging area for one row of block_mask bytes (2048 blocks and the alignment slack)
+constexpr int kSeqCap = 128;
+constexpr int kMaskWindow = 2048;
+constexpr int kMaskStage = kMaskWindow + 256;
 
 // Item header in LDS (16 ints).
 enum { H_HK = 0, H_QB, H_SUB, H_TOTAL, H_ROW_BEGIN, H_ROWS, H_KEY_BEGIN, H_Q_POS, H_SHIFT, H_PART, H_T0, H_SEQ, H_NKBLK, H_WORDS = 16 };
@@ -408,8 +420,11 @@ __device__ __forceinline__ int pack_tile(int pos, int valid) { return ((pos >> 4
 
 // Expands one item's kept-block bits into tile entries [chunk_base, chunk_base + kListCap) of
 // the item's tile sequence, written to list[0..); returns the item's total tile count.
-// Executed by one whole wavefront; `first_words`: lane i holds bit word i of the row.
-__device__ __forceinline__ int build_tile_list(int *list, int chunk_base, const uint32_t *row, int nwords, int kbs,
+// Executed by one whole wavefront; `first_words`: lane i holds bit word i of the row.  Rows longer than
+// 2048 blocks ask `more_words(window)` for the words window * 64 + lane (lane i: word window * 64 + i, zero
+// past the row's end), arrived and ready to use.
+template <typename MoreWords>
+__device__ __forceinline__ int build_tile_list(int *list, int chunk_base, MoreWords &&more_words, int nwords, int kbs,
                                                 FastDiv div_kbs, int kmax, uint32_t first_words, int lane) {
   if (kmax <= 0 || nwords <= 0) return 0;
   int total = 0;
@@ -426,10 +441,7 @@ __device__ __forceinline__ int build_tile_list(int *list, int chunk_base, const 
     for (int w2 = 0; w2 < nwords; w2 += 2) {
       if ((w2 >> 6) != window) {   // rows longer than 2048 blocks only
         window = w2 >> 6;
-        const int i = window * 64 + lane;
-        held = i < nwords ? row[i] : 0u;
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // wait here, not (for everything in flight) on the common path
-        asm volatile("" : "+v"(held));
+        held = more_words(window);
       }
       const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)held, w2 & 63);
       const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)held, (w2 + 1) & 63);   // nwords is even
@@ -457,10 +469,7 @@ __device__ __forceinline__ int build_tile_list(int *list, int chunk_base, const 
     auto word = [&](int w) -> uint32_t {
       if ((w >> 6) != window) {   // rows longer than 2048 blocks only
         window = w >> 6;
-        const int i = window * 64 + lane;
-        held = i < nwords ? row[i] : 0u;
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        asm volatile("" : "+v"(held));
+        held = more_words(window);
       }
       return (uint32_t)__builtin_amdgcn_readlane((int)held, w & 63);
     };
@@ -534,12 +543,15 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-template <int D, typename E, bool OUT32, int NW, bool EXTRAS>
+template <int D, typename E, bool OUT32, int NW, bool EXTRAS, bool FUSED>
 __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) {
   // OUT32: fp32 output (the fp32-input path; q/k/v are then fp16 staging copies)
   // EXTRAS: the clocked walk, the split over key blocks and the log-sum-exp output are compiled in.  The
   // plain call uses none of them, and its kernel is a tenth shorter without them (1-2 % faster: eight
   // wavefronts in different parts of a long kernel share one instruction cache).
+  // FUSED: the one-launch form.  No pre-pass has run: wavefront 0 derives an item's geometry from the
+  // sequence boundaries (kept in LDS) and its bit row from the item's own block_mask bytes, which it
+  // fetches into an LDS staging area one item ahead, where the other form fetches the prepared records.
   // NW: wavefronts (wave slots) of a workgroup, 4 or 8.  Eight are used when the q heads of a GQA group
   // and the 32-row slices of a q block give an item more than four wave slots: one workgroup per CU then
   // stages every K/V tile once for all of them instead of two workgroups staging it each.
@@ -556,6 +568,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
   char *lds_k = lds;
   int *lds_hdr = (int *)(lds + 4 * TILE_BYTES);     // [2][H_WORDS]
   int *lds_list = lds_hdr + 2 * H_WORDS;            // [2][kListCap]
+  int *lds_seq = lds_list + 2 * kListCap;           // FUSED: [4][kSeqCap] cu_q, cu_k, cu_num_q_block, cu_num_k_block
+  uint8_t *lds_mask = (uint8_t *)(lds_seq + 4 * kSeqCap);   // FUSED: [kMaskStage] block_mask bytes of the staged item
   auto hdr_word = [&](int c_, int i) { return __builtin_amdgcn_readfirstlane(lds_hdr[c_ * H_WORDS + i]); };
 
   const int lane = threadIdx.x & 63;
@@ -575,7 +589,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
   // counts the workgroup as done, and the workgroup that completes the count puts the queue counters
   // back to zero, so the next launch on this work description needs no preparation of its own.
   auto leave = [&]() {
-    if (wave != 0) return;
+    if (wave != 0 || p.one_each) return;
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this workgroup's last claim has returned
     if (lane == 0) {
       const uint32_t before = atomicAdd(&p.sched->done, 1u);
@@ -600,40 +614,159 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
     const int heads = v < p.nhead_k ? (p.nhead_k - v + 7) / 8 : 0;
     return (uint32_t)heads * (uint32_t)p.nqb * (uint32_t)p.nsub * (uint32_t)p.nparts;
   };
+  bool own_item_taken = false;   // one_each: this workgroup's only item has been handed out
   auto claim = [&]() -> uint32_t {   // the value is looked at an item later, so its latency is hidden
     uint32_t r = 0xffffffffu;
-    if (tries < 8) {
+    if (p.one_each) {
+      if (!own_item_taken) r = blockIdx.x;
+      own_item_taken = true;
+    } else if (tries < 8) {
       if (lane == 0) r = atomicAdd(&p.sched->qnext[(first_queue + tries) & 7], 1u);
     }
     return r;
   };
+  // (kv head, q block, slot group, part) of entry `claimed` of a head-major list that starts at kv head
+  // `head0` and holds every `head_step`-th head
+  auto decode_entry = [&](uint32_t claimed, int head0, int head_step) {
+    const uint32_t whole = fast_div(claimed, p.div_nparts);   // parts of one item are neighbours
+    st_part = (int)(claimed - whole * (uint32_t)p.nparts);
+    const uint32_t t = fast_div(whole, p.div_nsub);
+    st_sub = (int)(whole - t * (uint32_t)p.nsub);
+    const uint32_t h = fast_div(t, p.div_nqb);
+    st_hk = head0 + head_step * (int)h;
+    st_qb = p.nqb - 1 - (int)(t - h * (uint32_t)p.nqb);
+  };
+  // ---- one-launch form: geometry and mask bits without a pre-pass (wavefront 0)
+  const uint8_t *st_mrow = nullptr;   // staged item: address of the mask byte of its sequence's first k block
+  int st_nvis = 0, st_ms = 0;         // its k blocks below the causal bound; offset of the first one's byte in the staging area
+  // geometry of q block qb from the boundaries in LDS (uniform values); kb0: first global k block of its sequence.
+  // Consecutive items of a queue mostly belong to one sequence, so the last sequence's boundaries are kept.
+  SeqBounds seq_sb = {0, 0, 0, 0, 0, 0, 0};
+  int seq_qb_end = -1;      // q blocks [seq_sb.qb0, seq_qb_end) belong to the kept sequence (none at first)
+  bool seq_have = false;
+  auto fused_geometry = [&](int qb, int &kb0) -> QBlockInfo {
+    if (!(qb >= seq_sb.qb0 && qb < seq_qb_end)) {
+      int b = 0;   // sequences that start at or before qb, minus one
+      for (int base = 0; base < p.batch; base += 64) {
+        const int i = base + lane + 1;
+        const int first_qb = i <= p.batch ? lds_seq[2 * kSeqCap + i] : 0x7fffffff;
+        b += __builtin_popcountll(__builtin_amdgcn_ballot_w64(first_qb <= qb));
+      }
+      seq_have = b < p.batch;
+      seq_sb = SeqBounds{0, 0, 0, 0, 0, 0, 0};
+      seq_qb_end = -1;
+      if (seq_have) {
+        auto at = [&](int arr, int i) { return __builtin_amdgcn_readfirstlane(lds_seq[arr * kSeqCap + i]); };
+        seq_sb.q0 = at(0, b); seq_sb.q1 = at(0, b + 1);
+        seq_sb.k0 = at(1, b); seq_sb.k1 = at(1, b + 1);
+        seq_sb.qb0 = at(2, b); seq_qb_end = at(2, b + 1);
+        seq_sb.kb0 = at(3, b); seq_sb.kb1 = at(3, b + 1);
+      }
+    }
+    return q_block_geometry(qb, seq_have, seq_sb, p.qbs, p.kbs, p.causal, p.nkb_total, p.total_q, p.total_k, kb0);
+  };
+  const uint32_t lds_mask_addr = (uint32_t)(uintptr_t)HBSA_AS3(lds_mask);
+  // Requests the mask bytes of blocks [first, first + count), count <= kMaskWindow, of the row at `mrow`: whole
+  // aligned dwords, four bytes per lane, straight into the staging area (a dword that holds a byte of the
+  // row lies inside the mask's allocation).  Returns the offset of block `first`'s byte in the staging area.
+  auto mask_dma = [&](const uint8_t *mrow, int first, int count) -> int {
+    const uintptr_t a = (uintptr_t)(mrow + first);
+    const int sh = (int)(a & 3);
+    const char *base = (const char *)(a - sh);
+    const uint32_t last = (uint32_t)(sh + count - 1) & ~3u;   // offset of the last dword needed
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // what was read from the staging area before has arrived
+    for (uint32_t i = 0; i <= last; i += 256) {
+      const uint32_t off = min(i + 4u * (uint32_t)lane, last);   // every lane loads: lanes past the end repeat the last dword
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                   :
+                   : "s"(lds_mask_addr + i), "v"(off), "s"(base)
+                   : "memory", "m0");
+    }
+    return sh;
+  };
+  // bit words of the staged bytes: lane i gets word i (blocks 32 * i .. + 31 of the window; zero from `count` on)
+  auto staged_words = [&](int sh, int count) -> uint32_t {
+    uint32_t words = 0;
+    for (int w64 = 0; w64 * 64 < count; ++w64) {
+      const int j = w64 * 64 + lane;
+      const bool keep = j < count && lds_mask[sh + j] != 0;
+      const uint64_t bal = __builtin_amdgcn_ballot_w64(keep);
+      if (lane == 2 * w64) words = (uint32_t)bal;
+      if (lane == 2 * w64 + 1) words = (uint32_t)(bal >> 32);
+    }
+    return words;
+  };
+  // words of a later window of a row (rows longer than kMaskWindow blocks): fetched and waited for on the spot
+  auto fused_more_words = [&](const uint8_t *mrow, int nvis) {
+    return [&, mrow, nvis](int window) -> uint32_t {
+      const int first = window * kMaskWindow;
+      const int count = min(kMaskWindow, nvis - first);
+      if (count <= 0) return 0u;
+      const int sh = mask_dma(mrow, first, count);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      return staged_words(sh, count);
+    };
+  };
+  // the same for a prepared bit row in the workspace
+  auto prepared_more_words = [&](const uint32_t *row, int nwords) {
+    return [=](int window) -> uint32_t {
+      const int i = window * 64 + lane;
+      uint32_t held = i < nwords ? row[i] : 0u;
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // wait here, not (for everything in flight) on the common path
+      asm volatile("" : "+v"(held));
+      return held;
+    };
+  };
+
   // turn `pending` into the staged item (claiming again from the next queues when the one it
   // came from is exhausted) and start fetching the item's records
   auto stage = [&]() {
     uint32_t claimed = (uint32_t)__builtin_amdgcn_readfirstlane((int)pending);
     st_hk = -1;
-    while (tries < 8) {
-      const int v = (first_queue + tries) & 7;
-      if (claimed < queue_len(v)) {
-        const uint32_t whole = fast_div(claimed, p.div_nparts);   // parts of one item are neighbours in the queue
-        st_part = (int)(claimed - whole * (uint32_t)p.nparts);
-        const uint32_t t = fast_div(whole, p.div_nsub);
-        st_sub = (int)(whole - t * (uint32_t)p.nsub);
-        const uint32_t hq8 = fast_div(t, p.div_nqb);
-        st_hk = v + 8 * (int)hq8;
-        st_qb = p.nqb - 1 - (int)(t - hq8 * (uint32_t)p.nqb);
-        break;
+    if (p.one_each) {
+      if (claimed != 0xffffffffu) decode_entry(claimed, 0, 1);
+    } else {
+      while (tries < 8) {
+        const int v = (first_queue + tries) & 7;
+        if (claimed < queue_len(v)) {
+          decode_entry(claimed, v, 8);
+          break;
+        }
+        // This queue has run dry (the tail of the kernel).  Look at the other queues' counters first, all at
+        // once, and claim only from one that still shows work: a workgroup then ends after one load instead
+        // of seven failed claims in a row, each a round trip to a counter every other workgroup is hitting.
+        uint32_t seen = 0xffffffffu;
+        if (lane < 8) seen = __hip_atomic_load(&p.sched->qnext[(first_queue + lane) & 7], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        asm volatile("" : "+v"(seen));
+        const bool open = lane > tries && lane < 8 && seen < queue_len((first_queue + lane) & 7);
+        const uint64_t open_mask = __builtin_amdgcn_ballot_w64(open);
+        if (open_mask == 0) {
+          tries = 8;
+          break;
+        }
+        tries = __builtin_ctzll(open_mask);
+        uint32_t r = 0;
+        if (lane == 0) r = atomicAdd(&p.sched->qnext[(first_queue + tries) & 7], 1u);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        asm volatile("" : "+v"(r));
+        claimed = (uint32_t)__builtin_amdgcn_readfirstlane((int)r);
       }
-      if (++tries >= 8) break;
-      uint32_t r = 0;
-      if (lane == 0) r = atomicAdd(&p.sched->qnext[(first_queue + tries) & 7], 1u);
-      __builtin_amdgcn_s_waitcnt(0x0F70);   // only at the tail of the kernel, when a queue has run dry
-      asm volatile("" : "+v"(r));
-      claimed = (uint32_t)__builtin_amdgcn_readfirstlane((int)r);
     }
     if (st_hk >= 0) {
-      st_info = lane < 12 ? ((const uint32_t *)(p.info + st_qb))[lane] : 0u;
-      st_bits = lane < p.wpr ? p.bits[(((size_t)st_part * p.nhead_k + st_hk) * p.nqb + st_qb) * p.wpr + lane] : 0u;
+      if constexpr (FUSED) {
+        int kb0;
+        const QBlockInfo r = fused_geometry(st_qb, kb0);
+        st_info = (uint32_t)(lane == 0 ? r.row_begin : lane == 1 ? r.rows : lane == 2 ? r.key_begin : lane == 3 ? r.klen
+                             : lane == 4 ? r.q_pos : lane == 5 ? r.shift : lane == 6 ? r.nkblk : lane == 7 ? r.kmax
+                             : lane == 8 ? r.seq : 0);
+        st_nvis = min(r.nkblk, (int)fast_div((uint32_t)(r.kmax + p.kbs - 1), p.div_kbs));
+        st_mrow = p.mask + (int64_t)st_hk * p.ms_h + (int64_t)st_qb * p.ms_q + kb0;
+        st_ms = st_nvis > 0 ? mask_dma(st_mrow, 0, min(st_nvis, kMaskWindow)) : 0;
+      } else {
+        st_info = lane < 12 ? ((const uint32_t *)(p.info + st_qb))[lane] : 0u;
+        st_bits = lane < p.wpr ? p.bits[(((size_t)st_part * p.nhead_k + st_hk) * p.nqb + st_qb) * p.wpr + lane] : 0u;
+      }
     }
   };
   // expand the staged item into list `c` and write its header
@@ -643,9 +776,17 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
     if (st_hk >= 0) {
       const int nkblk = __builtin_amdgcn_readlane((int)st_info, 6);
       const int kmax = __builtin_amdgcn_readlane((int)st_info, 7);
-      total = build_tile_list(lds_list + c * kListCap, 0,
-                              p.bits + (((size_t)st_part * p.nhead_k + st_hk) * p.nqb + st_qb) * p.wpr,
-                              2 * ((nkblk + 63) >> 6), p.kbs, p.div_kbs, kmax, st_bits, lane);
+      if constexpr (FUSED) {
+        // the staged bytes arrived with the wait of a tile (or of the kernel's first lines) since stage()
+        st_bits = st_nvis > 0 ? staged_words(st_ms, min(st_nvis, kMaskWindow)) : 0u;
+        total = build_tile_list(lds_list + c * kListCap, 0, fused_more_words(st_mrow, st_nvis), 2 * ((st_nvis + 63) >> 6),
+                                p.kbs, p.div_kbs, kmax, st_bits, lane);
+      } else {
+        const int nwords = 2 * ((nkblk + 63) >> 6);
+        total = build_tile_list(lds_list + c * kListCap, 0,
+                                prepared_more_words(p.bits + (((size_t)st_part * p.nhead_k + st_hk) * p.nqb + st_qb) * p.wpr, nwords),
+                                nwords, p.kbs, p.div_kbs, kmax, st_bits, lane);
+      }
     }
     if (lane == 0) {
       hdr[H_HK] = st_hk; hdr[H_QB] = st_qb; hdr[H_SUB] = st_sub; hdr[H_TOTAL] = total; hdr[H_PART] = st_part;
@@ -749,8 +890,17 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
   };
 
   if (wave == 0) {
+    if constexpr (FUSED) {   // the sequences' boundaries, for fused_geometry()
+      for (int i = lane; i <= p.batch; i += 64) {
+        lds_seq[i] = p.cu_q[i];
+        lds_seq[kSeqCap + i] = p.cu_k[i];
+        lds_seq[2 * kSeqCap + i] = p.cu_nqb[i];
+        lds_seq[3 * kSeqCap + i] = p.cu_nkb[i];
+      }
+    }
     pending = claim();
     stage();
+    if constexpr (FUSED) __builtin_amdgcn_s_waitcnt(0x0F70);   // the first item's mask bytes
     build(0);
     note_item(0, hdr_word(0, H_TOTAL));
     pending = claim();
@@ -1201,11 +1351,23 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
       if (wave == 0) {
         // (the staged records now belong to a later item, so this item's are fetched again)
         const int qb = hdr_word(c, H_QB);
-        const QBlockInfo inf = p.info[qb];
-        const uint32_t *row = p.bits + (((size_t)cur_part * p.nhead_k + cur_hk) * p.nqb + qb) * p.wpr;
-        const int nwords = 2 * ((inf.nkblk + 63) >> 6);
-        (void)build_tile_list(lds_list + c * kListCap, chunk_base, row, nwords, p.kbs, p.div_kbs, inf.kmax,
-                              lane < nwords ? row[lane] : 0u, lane);
+        if constexpr (FUSED) {
+          int kb0;
+          const QBlockInfo inf = fused_geometry(qb, kb0);
+          const int nvis = min(inf.nkblk, (int)fast_div((uint32_t)(inf.kmax + p.kbs - 1), p.div_kbs));
+          auto more = fused_more_words(p.mask + (int64_t)cur_hk * p.ms_h + (int64_t)qb * p.ms_q + kb0, nvis);
+          const uint32_t first = more(0);
+          (void)build_tile_list(lds_list + c * kListCap, chunk_base, more, 2 * ((nvis + 63) >> 6), p.kbs, p.div_kbs, inf.kmax,
+                                first, lane);
+          // the staging area held the staged item's bytes: request them again (they arrive with the next tile's wait)
+          if (st_hk >= 0 && st_nvis > 0) st_ms = mask_dma(st_mrow, 0, min(st_nvis, kMaskWindow));
+        } else {
+          const QBlockInfo inf = p.info[qb];
+          const uint32_t *row = p.bits + (((size_t)cur_part * p.nhead_k + cur_hk) * p.nqb + qb) * p.wpr;
+          const int nwords = 2 * ((inf.nkblk + 63) >> 6);
+          (void)build_tile_list(lds_list + c * kListCap, chunk_base, prepared_more_words(row, nwords), nwords, p.kbs, p.div_kbs,
+                                inf.kmax, lane < nwords ? row[lane] : 0u, lane);
+        }
       }
       __syncthreads();
       {   // nothing is in flight here: fetch the chunk's first tile
@@ -1474,10 +1636,29 @@ int persistent_grid(const void *kernel, int lds_bytes, int threads) {
   return cus * per_cu;
 }
 
-template <int D, typename E, bool OUT32, int NW, bool EXTRAS>
+// The fields of FwdParams that follow from the call's shape and softmax_scale alone.
+void fill_shape(FwdParams &fp, int nhead_q, int nhead_k, int headdim, int num_q_block, int num_k_block, int q_block_size,
+                int k_block_size, int causal, float softmax_scale, bool f32_exact) {
+  fp.nhead_k = nhead_k;
+  fp.nqb = num_q_block; fp.ratio = nhead_q / nhead_k; fp.kbs = k_block_size; fp.wpr = words_per_row(num_k_block);
+  fp.causal = causal ? 1 : 0;
+  fp.wps = (q_block_size + kWaveRows - 1) / kWaveRows;
+  fp.nw = fwd_wavefronts(fp.ratio * fp.wps, headdim, f32_exact);
+  fp.nsub = (fp.ratio * fp.wps + fp.nw - 1) / fp.nw;
+  fp.div_nsub = make_fast_div((uint32_t)fp.nsub);
+  fp.div_nqb = make_fast_div((uint32_t)num_q_block);
+  fp.div_kbs = make_fast_div((uint32_t)k_block_size);
+  fp.q_sign = softmax_scale < 0.f ? 0x80008000u : 0u;
+  float c = std::fabs(softmax_scale) * kLog2e;
+  if (c < 1e-30f) c = 1e-30f;  // scale 0: uniform weights over the visible keys, and -inf * c stays -inf
+  fp.c = c;
+  fp.lag = kLazyRescaleLog2 / c;
+}
+
+template <int D, typename E, bool OUT32, int NW, bool EXTRAS, bool FUSED = false>
 int launch_fwd_nw(const FwdParams &fp, long long items, hipStream_t stream) {
-  constexpr int lds_bytes = 4 * kTileKeys * D * 2 + 2 * H_WORDS * 4 + 2 * kListCap * 4;
-  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS>);
+  constexpr int lds_bytes = 4 * kTileKeys * D * 2 + 2 * H_WORDS * 4 + 2 * kListCap * 4 + (FUSED ? 4 * kSeqCap * 4 + kMaskStage : 0);
+  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS, FUSED>);
   // workgroups that fit the current device at once; the attribute and the occupancy are per device
   static thread_local int resident_of[kMaxDevices] = {};
   int dev = 0;
@@ -1491,7 +1672,9 @@ int launch_fwd_nw(const FwdParams &fp, long long items, hipStream_t stream) {
     if (resident <= 0) return fail(HBSA_ERR_UNSUPPORTED, "could not size the persistent grid");
   }
   const int grid = (int)(items < resident ? items : resident);
-  hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS>), dim3(grid), dim3(NW * 64), lds_bytes, stream, fp);
+  FwdParams launch = fp;
+  launch.one_each = items <= resident ? 1 : 0;   // every item gets its own workgroup: no queues, no atomics
+  hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS, FUSED>), dim3(grid), dim3(NW * 64), lds_bytes, stream, launch);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail((int)e, "hbsa_fwd_kernel launch: %s", hipGetErrorString(e));
   return 0;
@@ -1504,6 +1687,14 @@ int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
       return extras ? launch_fwd_nw<D, E, OUT32, 8, true>(fp, items, stream) : launch_fwd_nw<D, E, OUT32, 8, false>(fp, items, stream);
   }
   return extras ? launch_fwd_nw<D, E, OUT32, 4, true>(fp, items, stream) : launch_fwd_nw<D, E, OUT32, 4, false>(fp, items, stream);
+}
+// the one-launch form (16-bit tensors, none of the extras)
+template <int D, typename E>
+int launch_fwd_fused(const FwdParams &fp, long long items, hipStream_t stream) {
+  if constexpr (D >= 64) {
+    if (fp.nw == 8) return launch_fwd_nw<D, E, false, 8, false, true>(fp, items, stream);
+  }
+  return launch_fwd_nw<D, E, false, 4, false, true>(fp, items, stream);
 }
 
 
@@ -1718,6 +1909,128 @@ int launch_fwd_f32(const FwdParams &fp, float c_signed, long long items, hipStre
 
 #include "hbsa_bwd.h"
 
+// ---- Device memory inside the library.  In host code the name of a __device__ array is only a handle; its
+// device address comes from hipGetSymbolAddress, once per device, and is what the kernels receive.  Every
+// GPU the library runs on holds its own copy of each array at its own address until the process ends.
+//
+// scratch: the work description of hbsa_fwd_static (hbsa_fwd without a workspace argument).
+// stream_sched: launch records (work-queue counters) of the one-launch form of hbsa_fwd, one per stream.  They
+// are zero when the library is loaded and every attention launch leaves its record at zero, so a call needs
+// no launch of its own to prepare one; calls on different streams use different records and may overlap.
+static __device__ __align__(256) unsigned char scratch[HBSA_STATIC_SCRATCH_BYTES];
+constexpr int kStreamSlots = 64;
+static __device__ __align__(256) unsigned char stream_sched[kStreamSlots * sizeof(Sched)];
+namespace {
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void **ptr) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail((int)e, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(HBSA_ERR_UNSUPPORTED, "device index above %d", kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) return fail(e != hipSuccess ? (int)e : HBSA_ERR_UNSUPPORTED, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+
+// The launch record of `stream` on the current device, nullptr when there is none to give (no device, the
+// lookup failed, or kStreamSlots other streams of this device have taken the records).
+struct StreamSlots {
+  char *base;
+  int used;
+  hipStream_t stream[kStreamSlots];
+};
+StreamSlots g_stream_slots[kMaxDevices] = {};
+Sched *stream_sched_of(hipStream_t stream) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  StreamSlots &t = g_stream_slots[dev];
+  if (t.base == nullptr) {
+    void *p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(stream_sched)) != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    t.base = (char *)p;
+  }
+  int i = 0;
+  while (i < t.used && t.stream[i] != stream) ++i;
+  if (i == t.used) {
+    if (t.used == kStreamSlots) return nullptr;
+    t.stream[t.used++] = stream;
+  }
+  return (Sched *)(t.base + (size_t)i * sizeof(Sched));
+}
+
+// The one-launch form of the forward is used when it applies (see hbsa_set_onepass in the header).
+int g_onepass = [] {
+  const char *e = std::getenv("HBSATTN_AMD_ONEPASS");
+  return e != nullptr && e[0] == '0' && e[1] == 0 ? 0 : 1;
+}();
+
+// The launch record a call would use in the one-launch form, nullptr when the form does not apply to it.
+Sched *onepass_record(int32_t dtype, int32_t batch, int32_t total_k, int32_t headdim, int32_t num_k_block, int32_t k_block_size,
+                      int64_t mask_kblk_stride, long long items, hipStream_t st) {
+  if (!g_onepass || (dtype != HBSA_DTYPE_BF16 && dtype != HBSA_DTYPE_F16)) return nullptr;
+  if (mask_kblk_stride != 1 || batch < 1 || batch >= kSeqCap) return nullptr;
+  if (items <= 0 || items > 0x7fffffffLL) return nullptr;
+  if (split_parts(items, num_k_block) > 1) return nullptr;
+  if (!g_deterministic && k_block_size % kTileKeys == 0 && 2ll * total_k * headdim * 2 >= g_walk_min_bytes) return nullptr;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &capturing) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  if (capturing != hipStreamCaptureStatusNone) return nullptr;
+  return stream_sched_of(st);
+}
+
+constexpr int kNotOnePass = 0x7fffffff;   // try_onepass: the call has to take the two-launch path
+
+// hbsa_fwd as ONE launch: the attention kernel's scheduler reads the sequence boundaries and the mask bytes
+// itself.  Arguments are those of hbsa_fwd, already validated.  Returns kNotOnePass when the form does not
+// apply: fp32 tensors, a mask whose k block stride is not 1, more than kSeqCap - 1 sequences, work that
+// would be split over key blocks or walk by the clock, a stream that is being captured into a graph (the
+// graph could be replayed on any stream, while the launch record belongs to this one), no launch record left.
+int try_onepass(const void *q, const void *k, const void *v, void *out, const int32_t *cu_q_seqlens,
+                const int32_t *cu_k_seqlens, const uint8_t *block_mask, const int32_t *cu_num_q_block,
+                const int32_t *cu_num_k_block, int32_t dtype, int32_t batch, int32_t total_q, int32_t total_k, int32_t nhead_q,
+                int32_t nhead_k, int32_t headdim, int32_t num_q_block, int32_t num_k_block, int32_t q_block_size,
+                int32_t k_block_size, int32_t causal, float softmax_scale, const int64_t *strides, hipStream_t st) {
+  FwdParams fp;
+  std::memset(&fp, 0, sizeof(fp));
+  fill_shape(fp, nhead_q, nhead_k, headdim, num_q_block, num_k_block, q_block_size, k_block_size, causal, softmax_scale, false);
+  const long long items = (long long)nhead_k * num_q_block * fp.nsub;
+  Sched *sched = onepass_record(dtype, batch, total_k, headdim, num_k_block, k_block_size, strides[10], items, st);
+  if (sched == nullptr) return kNotOnePass;
+
+  fp.q = (const char *)q; fp.k = (const char *)k; fp.v = (const char *)v; fp.out = (char *)out;
+  fp.sched = sched;
+  fp.q_s = strides[0] * 2; fp.q_h = strides[1] * 2; fp.k_s = strides[2] * 2; fp.k_h = strides[3] * 2;
+  fp.v_s = strides[4] * 2; fp.v_h = strides[5] * 2; fp.o_s = strides[6] * 2; fp.o_h = strides[7] * 2;
+  fp.nparts = 1;
+  fp.div_nparts = make_fast_div(1u);
+  fp.total_q = total_q; fp.nhead_q = nhead_q;
+  fp.cu_q = cu_q_seqlens; fp.cu_k = cu_k_seqlens; fp.cu_nqb = cu_num_q_block; fp.cu_nkb = cu_num_k_block;
+  fp.mask = block_mask; fp.ms_h = strides[8]; fp.ms_q = strides[9];
+  fp.batch = batch; fp.nkb_total = num_k_block; fp.total_k = total_k; fp.qbs = q_block_size;
+  const bool bf = dtype == HBSA_DTYPE_BF16;
+  switch (headdim) {
+    case 32: return bf ? launch_fwd_fused<32, ElemBF16>(fp, items, st) : launch_fwd_fused<32, ElemF16>(fp, items, st);
+    case 64: return bf ? launch_fwd_fused<64, ElemBF16>(fp, items, st) : launch_fwd_fused<64, ElemF16>(fp, items, st);
+    default: return bf ? launch_fwd_fused<128, ElemBF16>(fp, items, st) : launch_fwd_fused<128, ElemF16>(fp, items, st);
+  }
+}
+}  // namespace
+
 extern "C" {
 
 int hbsa_abi_version(void) { return HBSA_ABI_VERSION; }
@@ -1725,6 +2038,25 @@ int hbsa_abi_version(void) { return HBSA_ABI_VERSION; }
 int hbsa_set_deterministic(int on) {
   const int previous = g_deterministic;
   g_deterministic = on ? 1 : 0;
+  return previous;
+}
+
+int hbsa_fwd_launches(int32_t dtype, int32_t batch, int32_t total_k, int32_t nhead_q, int32_t nhead_k, int32_t headdim,
+                      int32_t num_q_block, int32_t num_k_block, int32_t q_block_size, int32_t k_block_size,
+                      int64_t mask_kblk_stride, void *stream) {
+  if (nhead_k <= 0 || nhead_q <= 0 || nhead_q % nhead_k != 0 || num_q_block <= 0 || num_k_block <= 0 || q_block_size <= 0 ||
+      k_block_size <= 0 || (headdim != 32 && headdim != 64 && headdim != 128))
+    return 2;
+  const int ratio = nhead_q / nhead_k, wps = (q_block_size + kWaveRows - 1) / kWaveRows;
+  const int nw = fwd_wavefronts(ratio * wps, headdim, false);
+  const long long items = (long long)nhead_k * num_q_block * ((ratio * wps + nw - 1) / nw);
+  return onepass_record(dtype, batch, total_k, headdim, num_k_block, k_block_size, mask_kblk_stride, items,
+                        (hipStream_t)stream) != nullptr ? 1 : 2;
+}
+
+int hbsa_set_onepass(int on) {
+  const int previous = g_onepass;
+  g_onepass = on ? 1 : 0;
   return previous;
 }
 
@@ -1902,19 +2234,8 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
     fp.q_s = strides[0] * es; fp.q_h = strides[1] * es; fp.k_s = strides[2] * es; fp.k_h = strides[3] * es;
     fp.v_s = strides[4] * es; fp.v_h = strides[5] * es; fp.o_s = strides[6] * es; fp.o_h = strides[7] * es;
   }
-  fp.nqb = num_q_block; fp.ratio = nhead_q / nhead_k; fp.kbs = k_block_size; fp.wpr = words_per_row(num_k_block);
-  fp.causal = causal ? 1 : 0;
-  fp.wps = (q_block_size + kWaveRows - 1) / kWaveRows;
-  fp.nw = fwd_wavefronts(fp.ratio * fp.wps, headdim, f32_exact);
-  fp.nsub = (fp.ratio * fp.wps + fp.nw - 1) / fp.nw;
-  fp.div_nsub = make_fast_div((uint32_t)fp.nsub);
-  fp.div_nqb = make_fast_div((uint32_t)num_q_block);
-  fp.div_kbs = make_fast_div((uint32_t)k_block_size);
-  fp.q_sign = softmax_scale < 0.f ? 0x80008000u : 0u;
-  float c = std::fabs(softmax_scale) * kLog2e;
-  if (c < 1e-30f) c = 1e-30f;  // scale 0: uniform weights over the visible keys, and -inf * c stays -inf
-  fp.c = c;
-  fp.lag = kLazyRescaleLog2 / c;
+  fill_shape(fp, nhead_q, nhead_k, headdim, num_q_block, num_k_block, q_block_size, k_block_size, causal, softmax_scale,
+             f32_exact);
   const long long items = (long long)nhead_k * num_q_block * fp.nsub;
   if (items > 0x7fffffffLL) return fail(HBSA_ERR_UNSUPPORTED, "too many work items (%lld)", items);
   // split over key blocks when the items cannot fill the device and the caller's workspace has the room
@@ -1967,13 +2288,16 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
   }
 }
 
-int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32_t *cu_q_seqlens,
+}  // extern "C"
+namespace {
+// hbsa_fwd, with the one-launch form allowed or not
+int fwd_call(const void *q, const void *k, const void *v, void *out, const int32_t *cu_q_seqlens,
              const int32_t *cu_k_seqlens, const uint8_t *block_mask, const int32_t *q_block_to_batch,
              const int32_t *cu_num_q_block, const int32_t *cu_num_k_block, void *workspace,
              size_t workspace_bytes, int32_t dtype, int32_t batch, int32_t total_q, int32_t total_k,
              int32_t nhead_q, int32_t nhead_k, int32_t headdim, int32_t num_q_block, int32_t num_k_block,
              int32_t q_block_size, int32_t k_block_size, int32_t causal, float softmax_scale,
-             const int64_t *strides, void *stream) {
+             const int64_t *strides, void *stream, bool allow_onepass) {
   g_err[0] = 0;
   if (total_q == 0 || num_q_block == 0 || nhead_q == 0) return 0;
   if (!strides) return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer argument");
@@ -1989,11 +2313,26 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
     return fail(HBSA_ERR_INVALID_ARGUMENT, "q/k/v/out must be 16-byte aligned");
   if (int rc = check_strides(strides, dtype == HBSA_DTYPE_F32 || dtype == HBSA_DTYPE_F32_STAGED16)) return rc;
+  if (batch < 0 || num_q_block < 0 || num_k_block < 0 || total_q < 0 || total_k < 0)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "negative size");
+  if (!cu_q_seqlens || !cu_k_seqlens || !block_mask || !q_block_to_batch || !cu_num_q_block || !cu_num_k_block)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer argument");
+  if (q_block_size <= 0 || k_block_size <= 0 || q_block_size % 16 || k_block_size % 16)
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "q_block_size (%d) and k_block_size (%d) must be positive multiples of 16",
+                q_block_size, k_block_size);
+  if (num_k_block <= 0 || total_k <= 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "no keys");
+  if (nhead_k > 65535) return fail(HBSA_ERR_UNSUPPORTED, "nhead_k %d > 65535", nhead_k);
+  if (allow_onepass) {
+    const int one = try_onepass(q, k, v, out, cu_q_seqlens, cu_k_seqlens, block_mask, cu_num_q_block, cu_num_k_block, dtype,
+                                batch, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block, num_k_block, q_block_size,
+                                k_block_size, causal, softmax_scale, strides, (hipStream_t)stream);
+    if (one != kNotOnePass) return one;
+  }
   {
     const size_t need = hbsa_fwd_workspace_bytes_dtype(dtype, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
                                                        num_k_block);
-    if (workspace_bytes < need)
-      return fail(HBSA_ERR_WORKSPACE_TOO_SMALL, "workspace %zu bytes < required %zu", workspace_bytes, need);
+    if (!workspace || workspace_bytes < need)
+      return fail(HBSA_ERR_WORKSPACE_TOO_SMALL, "workspace %zu bytes < required %zu", workspace ? workspace_bytes : (size_t)0, need);
   }
   int rc = hbsa_fwd_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_to_batch, cu_num_q_block, cu_num_k_block,
                             workspace, workspace_bytes, batch, nhead_k, num_q_block, num_k_block, q_block_size,
@@ -2002,34 +2341,32 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32
   return hbsa_fwd_run(q, k, v, out, workspace, workspace_bytes, dtype, total_q, total_k, nhead_q, nhead_k, headdim,
                       num_q_block, num_k_block, q_block_size, k_block_size, causal, softmax_scale, strides, stream);
 }
-
-// ---- hbsa_fwd without a workspace argument: the work description lives in this array.  Every GPU
-// the library runs on holds its own copy at its own address until the process ends.  In host code
-// the array's name is only a handle; its device address comes from hipGetSymbolAddress, once per
-// device, and is what the kernels receive.
-}  // extern "C"
-static __device__ __align__(256) unsigned char scratch[HBSA_STATIC_SCRATCH_BYTES];
-namespace {
-std::mutex g_scratch_mutex;
-void *g_scratch_ptr[kMaxDevices] = {};
-
-int static_scratch(void **ptr) {
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return fail((int)e, "hipGetDevice: %s", hipGetErrorString(e));
-  if (dev < 0 || dev >= kMaxDevices) return fail(HBSA_ERR_UNSUPPORTED, "device index above %d", kMaxDevices - 1);
-  std::lock_guard<std::mutex> lock(g_scratch_mutex);
-  if (g_scratch_ptr[dev] == nullptr) {
-    void *p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e != hipSuccess || p == nullptr) return fail(e != hipSuccess ? (int)e : HBSA_ERR_UNSUPPORTED, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
-    g_scratch_ptr[dev] = p;
-  }
-  *ptr = g_scratch_ptr[dev];
-  return 0;
-}
 }  // namespace
 extern "C" {
+
+int hbsa_fwd(const void *q, const void *k, const void *v, void *out, const int32_t *cu_q_seqlens,
+             const int32_t *cu_k_seqlens, const uint8_t *block_mask, const int32_t *q_block_to_batch,
+             const int32_t *cu_num_q_block, const int32_t *cu_num_k_block, void *workspace,
+             size_t workspace_bytes, int32_t dtype, int32_t batch, int32_t total_q, int32_t total_k,
+             int32_t nhead_q, int32_t nhead_k, int32_t headdim, int32_t num_q_block, int32_t num_k_block,
+             int32_t q_block_size, int32_t k_block_size, int32_t causal, float softmax_scale,
+             const int64_t *strides, void *stream) {
+  return fwd_call(q, k, v, out, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_to_batch, cu_num_q_block, cu_num_k_block,
+                  workspace, workspace_bytes, dtype, batch, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
+                  num_k_block, q_block_size, k_block_size, causal, softmax_scale, strides, stream, true);
+}
+
+int hbsa_fwd_v(const void *const *ptrs, size_t workspace_bytes, const int32_t *sizes, float softmax_scale,
+               const int64_t *strides, void *stream) {
+  if (!ptrs || !sizes) {
+    g_err[0] = 0;
+    return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer argument");
+  }
+  return fwd_call(ptrs[0], ptrs[1], ptrs[2], (void *)ptrs[3], (const int32_t *)ptrs[4], (const int32_t *)ptrs[5],
+                  (const uint8_t *)ptrs[6], (const int32_t *)ptrs[7], (const int32_t *)ptrs[8], (const int32_t *)ptrs[9],
+                  (void *)ptrs[10], workspace_bytes, sizes[0], sizes[1], sizes[2], sizes[3], sizes[4], sizes[5], sizes[6], sizes[7],
+                  sizes[8], sizes[9], sizes[10], sizes[11], softmax_scale, strides, stream, true);
+}
 
 int hbsa_fwd_static(const void *q, const void *k, const void *v, void *out, const int32_t *cu_q_seqlens,
                     const int32_t *cu_k_seqlens, const uint8_t *block_mask, const int32_t *q_block_to_batch,
@@ -2047,9 +2384,10 @@ int hbsa_fwd_static(const void *q, const void *k, const void *v, void *out, cons
                 (size_t)HBSA_STATIC_SCRATCH_BYTES);
   void *ws = nullptr;
   if (int rc = static_scratch(&ws)) return rc;
-  return hbsa_fwd(q, k, v, out, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_to_batch, cu_num_q_block, cu_num_k_block, ws,
+  // (always the pre-pass and the attention kernel on the static array: this form may be captured into a graph)
+  return fwd_call(q, k, v, out, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_to_batch, cu_num_q_block, cu_num_k_block, ws,
                   (size_t)HBSA_STATIC_SCRATCH_BYTES, dtype, batch, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
-                  num_k_block, q_block_size, k_block_size, causal, softmax_scale, strides, stream);
+                  num_k_block, q_block_size, k_block_size, causal, softmax_scale, strides, stream, false);
 }
 
 size_t hbsa_bwd_workspace_bytes(int32_t total_q, int32_t nhead_q) {

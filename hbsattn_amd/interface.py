@@ -48,6 +48,8 @@ def set_deterministic(on: bool) -> bool:
     the library is loaded), very large problems order the walk by a clock shared between workgroups,
     which saves HBM traffic and lets the last bits of the result depend on timing.  Returns the previous
     setting."""
+    _needs_workspace.clear()   # which calls run as one launch depends on the mode
+    _direct_plans.clear()
     return bool(_lib.load().hbsa_set_deterministic(1 if on else 0))
 
 
@@ -365,20 +367,122 @@ def _cached_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_bloc
     return prepared
 
 
+try:
+    _raw_stream = torch._C._cuda_getCurrentRawStream     # the current stream's handle without building a Stream object
+except AttributeError:                                    # pragma: no cover
+    def _raw_stream(index):
+        return torch.cuda.current_stream(index).cuda_stream
+
+# Shapes for which hbsa_fwd asked for a workspace (its one-launch form does not apply to them): those go
+# straight to the prepare + run path instead of asking again on every call.
+_needs_workspace = set()
+
+
+def set_onepass(on: bool) -> bool:
+    """The library's one-launch form of the forward (``hbsa_set_onepass``), on by default; returns the
+    previous setting."""
+    _needs_workspace.clear()
+    _direct_plans.clear()
+    return bool(_lib.load().hbsa_set_onepass(1 if on else 0))
+
+
+# Per-shape state of the direct path: the size and stride arrays of a call whose tensors are all contiguous
+# are functions of the shapes alone, so they are built once per shape, together with the pointer array
+# that every call refills (``hbsa_fwd_v``).
+_direct_plans = {}
+_I32 = torch.int32
+
+
+def _forward_direct(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, softmax_scale,
+                    num_q_block, q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block):
+    """``hbsa_fwd`` without a workspace: one launch when the library's one-launch form applies, ``None``
+    when the call has to go through ``hbsa_prepare`` / ``hbsa_run``.  This is the path of a plain forward
+    call, so it does as little on the host as the checks allow: contiguous bf16 / fp16 tensors with a
+    native head dim and int32 metadata; everything else takes the general path, which also raises
+    the errors."""
+    dtype = q.dtype
+    if dtype is not torch.bfloat16 and dtype is not torch.float16:
+        return None
+    try:
+        total_q, nhead_q, headdim = q.shape
+        total_k, nhead_k, _ = k.shape
+        n_seq, = cu_q_seqlens.shape
+    except (ValueError, AttributeError):
+        return None
+    key = (total_q, total_k, nhead_q, nhead_k, headdim, num_q_block, num_k_block, q_block_size, k_block_size, causal, n_seq,
+           dtype)
+    plan = _direct_plans.get(key)
+    if plan is None:
+        if headdim not in _NATIVE_HEADDIMS or total_q == 0 or total_k == 0 or n_seq < 2 or key in _needs_workspace:
+            return None
+        _check_block_sizes(q_block_size, k_block_size)
+        strides = (ctypes.c_int64 * 11)(nhead_q * headdim, headdim, nhead_k * headdim, headdim, nhead_k * headdim, headdim,
+                                        nhead_q * headdim, headdim, num_q_block * num_k_block, num_k_block, 1)
+        sizes = (ctypes.c_int32 * 12)(_DTYPE_CODES[dtype], n_seq - 1, total_q, total_k, nhead_q, nhead_k, headdim, num_q_block,
+                                      num_k_block, q_block_size, k_block_size, 1 if causal else 0)
+        ptrs = (ctypes.c_void_p * 11)()
+        plan = (ptrs, ctypes.addressof(ptrs), ctypes.addressof(sizes), ctypes.addressof(strides), sizes, strides,
+                _lib.load().hbsa_fwd_v_locked)
+        if len(_direct_plans) > 4096:
+            _direct_plans.clear()
+        _direct_plans[key] = plan
+    dev = q.device
+    index = dev.index
+    if not (k.dtype is dtype and v.dtype is dtype and v.shape == k.shape and k.device == dev and v.device == dev
+            and q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and block_mask.is_contiguous()):
+        return None
+    for t, n in ((cu_q_seqlens, n_seq), (cu_k_seqlens, n_seq), (cu_num_q_block, n_seq), (cu_num_k_block, n_seq),
+                 (q_block_to_batch, num_q_block)):
+        if not (isinstance(t, torch.Tensor) and t.dtype is _I32 and t.get_device() == index and t.numel() == n
+                and t.is_contiguous()):
+            return None
+    qp, kp, vp = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    if (qp | kp | vp) & 15:
+        return None
+    if index != torch.cuda.current_device():
+        with torch.cuda.device(dev):
+            return _forward_direct(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal,
+                                   softmax_scale, num_q_block, q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block)
+    scale = float(softmax_scale) if softmax_scale is not None else headdim ** -0.5
+    out = torch.empty_like(q)
+    ptrs = plan[0]
+    ptrs[0] = qp; ptrs[1] = kp; ptrs[2] = vp; ptrs[3] = out.data_ptr()
+    ptrs[4] = cu_q_seqlens.data_ptr(); ptrs[5] = cu_k_seqlens.data_ptr(); ptrs[6] = block_mask.data_ptr()
+    ptrs[7] = q_block_to_batch.data_ptr(); ptrs[8] = cu_num_q_block.data_ptr(); ptrs[9] = cu_num_k_block.data_ptr()
+    rc = plan[6](plan[1], 0, plan[2], scale, plan[3], _raw_stream(index))
+    if rc == 0:
+        return out
+    if rc == _lib.ERR_WORKSPACE_TOO_SMALL:   # nothing was launched: this call takes the two-launch path
+        if not torch.cuda.is_current_stream_capturing():   # ... and so will every call of this shape
+            if len(_needs_workspace) > 4096:
+                _needs_workspace.clear()
+            _needs_workspace.add(key)
+            _direct_plans.pop(key, None)
+        return None
+    raise RuntimeError(f"hbsa_fwd failed (code {rc}): {_lib.last_error()}")
+
+
 def hbsa_forward(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, softmax_scale,
                  num_q_block, q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, ctx=None) -> torch.Tensor:
-    """Host launcher: checks, scratch allocation, pre-pass (skipped when the same mask and sequence
-    boundaries were prepared by a recent call) and attention kernel through the C ABI.
+    """Host launcher: checks, then either ``hbsa_fwd`` directly (a plain forward call: one launch when the
+    library's one-launch form applies) or scratch allocation, pre-pass (skipped when the same mask and
+    sequence boundaries were prepared by a recent call) and attention kernel.
     No device synchronisation happens here."""
     if not q.is_cuda:
         raise RuntimeError("hbsattn_amd runs on MI355X only: q/k/v must be CUDA(HIP) tensors; there is no CPU path")
     if block_mask.device != q.device:
         raise RuntimeError("q, k, v and block_mask must live on the same device")
     assert q.shape[1] % k.shape[1] == 0, "nhead_q must be divisible by nhead_k (for GQA)"
+    wants_grad = ctx is not None and any(ctx.needs_input_grad[:3]) and backward_supported(q)
+    if not wants_grad and _prepared_cache_size == 0:
+        out = _forward_direct(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal,
+                              softmax_scale, num_q_block, q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block)
+        if out is not None:
+            return out
     run_shape = (q.dtype, q.shape[0], k.shape[0], q.shape[1], q.shape[2]) if q.dim() == 3 and k.dim() == 3 else None
     prepared = _cached_prepare(cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, num_q_block,
                                q_block_to_batch, cu_num_q_block, num_k_block, cu_num_k_block, run_shape)
-    if ctx is not None and any(ctx.needs_input_grad[:3]) and backward_supported(q):
+    if wants_grad:
         # keep what the backward needs: the log-sum-exp, the output and the prepared mask
         out, lse = hbsa_run(q, k, v, prepared, softmax_scale, return_lse=True)
         ctx.save_for_backward(q, k, v, out, lse)
@@ -428,4 +532,16 @@ class _HBSAttentionFunction(torch.autograd.Function):
         return (dq, dk, dv) + (None,) * 16
 
 
-HBSAttention = _HBSAttentionFunction.apply
+def HBSAttention(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size, causal, softmax_scale,
+                 tile_mode="auto", num_q_block=None, cu_q_block=None, q_block_to_batch=None, cu_num_q_block=None,
+                 num_k_block=None, cu_k_block=None, k_block_to_batch=None, cu_num_k_block=None):
+    """Same call as the reference's ``HBSAttention`` (``_HBSAttentionFunction.apply``, reference
+    ``hbsattn/hbsa_interface.py:35``).  The autograd machinery is entered only when a gradient can be asked
+    for; a plain forward call goes straight to the launcher."""
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        return _HBSAttentionFunction.apply(q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size,
+                                           causal, softmax_scale, tile_mode, num_q_block, cu_q_block, q_block_to_batch,
+                                           cu_num_q_block, num_k_block, cu_k_block, k_block_to_batch, cu_num_k_block)
+    return _HBSAttentionFunction.forward(None, q, k, v, cu_q_seqlens, cu_k_seqlens, block_mask, q_block_size, k_block_size,
+                                         causal, softmax_scale, tile_mode, num_q_block, cu_q_block, q_block_to_batch,
+                                         cu_num_q_block, num_k_block, cu_k_block, k_block_to_batch, cu_num_k_block)

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define HBSA_ABI_VERSION 5
+#define HBSA_ABI_VERSION 6
 
 /* element types of q/k/v/out (reference: dtype follows the input tensors,
  * hbsattn/fwd_triton_auto_tile_size.py:272) */
@@ -66,6 +66,15 @@ const char *hbsa_last_error(void);
  * their last bits (the error against an exact evaluation is unchanged).
  */
 int hbsa_set_deterministic(int on);
+
+int hbsa_set_onepass(int on);   /* see hbsa_fwd */
+
+/* Launches an hbsa_fwd call with these sizes would make on `stream` right now: 1 when its one-launch form
+ * applies (the call then needs no workspace), else 2 (pre-pass and attention kernel; more for
+ * HBSA_DTYPE_F32_STAGED16 and for work split over key blocks).  Host-side only, nothing is launched. */
+int hbsa_fwd_launches(int32_t dtype, int32_t batch, int32_t total_k, int32_t nhead_q, int32_t nhead_k,
+                      int32_t headdim, int32_t num_q_block, int32_t num_k_block,
+                      int32_t q_block_size, int32_t k_block_size, int64_t mask_kblk_stride, void *stream);
 
 /* Size (K + V bytes of one kv head) from which the clocked walk above is used; a negative value only
  * reads the setting.  Returns the previous value. */
@@ -144,7 +153,23 @@ size_t hbsa_fwd_split_workspace_bytes(int32_t total_q, int32_t nhead_q, int32_t 
  *   softmax_scale  already resolved (the caller substitutes headdim**-0.5 for None)
  *   strides     int64[11] = { q_tok, q_head, k_tok, k_head, v_tok, v_head,
  *                             out_tok, out_head, mask_head, mask_qblk, mask_kblk }
- *   workspace   >= hbsa_fwd_workspace_bytes_dtype(...) bytes, 256-byte aligned
+ *   workspace   >= hbsa_fwd_workspace_bytes_dtype(...) bytes, 256-byte aligned; may be NULL (with
+ *               workspace_bytes 0) for a call that runs as one launch, see below
+ *
+ * Launches.  In general the call is two launches, hbsa_fwd_prepare's pre-pass (mask bytes and sequence
+ * boundaries -> a compact work description in `workspace`) and the attention kernel.  A call on bf16 or
+ * fp16 tensors is ONE launch, and does not touch `workspace`, when the attention kernel's scheduler can
+ * read the boundaries and the mask bytes itself: mask_kblk stride 1, at most 127 sequences, work that
+ * would neither be split over key blocks (hbsa_fwd_split_workspace_bytes) nor use the clocked walk,
+ * `stream` not being captured into a graph, and fewer than 64 other streams of the device having made such
+ * calls.  The launch record (work-queue counters) of that form lives in device memory inside the library,
+ * one record per stream, so calls on different streams may overlap; it replaces the reference kernel's
+ * per-program scan of the mask (reference hbsattn/fwd_triton_auto_tile_size.py:153-164) and the
+ * launcher's two host synchronisations (:276-277) with nothing at all.  Results are bitwise those of the
+ * two-launch path.  A call that cannot run as one launch and has no (or too small a) workspace returns
+ * HBSA_ERR_WORKSPACE_TOO_SMALL before anything is launched.  hbsa_set_onepass(0) switches the form off
+ * (process-wide; returns the previous setting; the environment variable HBSATTN_AMD_ONEPASS=0 does the same
+ * when the library is loaded).
  *
  * Supported: headdim in {32, 64, 128}; q_block_size, k_block_size positive multiples
  * of 16; nhead_q % nhead_k == 0; every sequence length >= 1.  Query rows with no
@@ -162,6 +187,19 @@ int hbsa_fwd(const void *q, const void *k, const void *v, void *out,
              int32_t q_block_size, int32_t k_block_size,
              int32_t causal, float softmax_scale,
              const int64_t *strides, void *stream);
+
+/*
+ * hbsa_fwd with its arguments in arrays, for bindings that pay per argument (Python's ctypes spends more
+ * host time on hbsa_fwd's 27 arguments than a small problem's kernel runs).  Same checks, launches and
+ * results as hbsa_fwd:
+ *   ptrs   host array of 11 pointers = { q, k, v, out, cu_q_seqlens, cu_k_seqlens, block_mask,
+ *          q_block_to_batch, cu_num_q_block, cu_num_k_block, workspace }
+ *   sizes  host array of 12 ints = { dtype, batch, total_q, total_k, nhead_q, nhead_k, headdim,
+ *          num_q_block, num_k_block, q_block_size, k_block_size, causal }
+ * Both arrays are read during the call only.
+ */
+int hbsa_fwd_v(const void *const *ptrs, size_t workspace_bytes, const int32_t *sizes, float softmax_scale,
+               const int64_t *strides, void *stream);
 
 /*
  * hbsa_fwd for callers that cannot allocate device memory or pass a workspace: code under HIP

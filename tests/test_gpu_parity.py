@@ -295,12 +295,82 @@ def test_combined_c_entry_point_matches_operator_and_oracle(dtype):
 def test_combined_c_entry_point_rejects_bad_arguments_without_launching():
     w = make_problem(seed=22, q_lens=[256], k_lens=[256], hq=2, hk=2, d=64, qbs=64, kbs=64, keep=0.5, diag=True,
                      causal=False, scale=None)
-    rc, out, msg = _call_hbsa_fwd(w, workspace_bytes=16)
+    from hbsattn_amd import _lib
+    lib = _lib.load()
+    one = lib.hbsa_set_onepass(0)            # the two-launch path needs its workspace
+    try:
+        rc, out, msg = _call_hbsa_fwd(w, workspace_bytes=16)
+    finally:
+        lib.hbsa_set_onepass(one)
     assert rc == -3 and "workspace" in msg
     assert torch.isnan(out.float()).all()
+    rc, out, msg = _call_hbsa_fwd(w, workspace_bytes=0)   # as one launch the call uses no workspace
+    assert rc == 0 and torch.equal(out, _run(w))
     rc, out, msg = _call_hbsa_fwd(w, headdim=48)
     assert rc == -2 and "headdim" in msg
     assert torch.isnan(out.float()).all()
+
+
+def _launches(w):
+    from hbsattn_amd import _lib
+    from hbsattn_amd.interface import _dtype_code
+    return _lib.load().hbsa_fwd_launches(_dtype_code(w.q.dtype), len(w.cu_q) - 1, w.k.shape[0], w.q.shape[1], w.k.shape[1],
+                                         w.q.shape[2], w.q_meta[0], w.k_meta[0], w.q_block_size, w.k_block_size,
+                                         w.block_mask.stride(2), torch.cuda.current_stream().cuda_stream)
+
+
+@pytest.mark.parametrize("spec,launches", [
+    (dict(q_lens=[1100, 300, 2048], k_lens=[1500, 300, 2048], hq=16, hk=8, d=64, qbs=64, kbs=64, keep=0.3, causal=True), 1),
+    (dict(q_lens=[4096, 1536, 2048], k_lens=[4096, 3000, 2048], hq=16, hk=16, d=128, qbs=128, kbs=128, keep=0.25, causal=False), 1),
+    (dict(q_lens=[3000, 5120, 777], k_lens=[6000, 5120, 4100], hq=16, hk=2, d=64, qbs=80, kbs=48, keep=0.5, causal=True), 1),
+    (dict(q_lens=[256, 0, 0, 64, 0, 384], k_lens=[512, 128, 0, 256, 128, 640], hq=4, hk=4, d=128, qbs=128, kbs=128, keep=0.5, causal=True), 1),
+    (dict(q_lens=[700, 600], k_lens=[40000, 900], hq=24, hk=12, d=32, qbs=32, kbs=16, keep=0.4, causal=True), 1),      # rows beyond one staging window
+    (dict(q_lens=[1600, 1200], k_lens=[150000, 3000], hq=16, hk=8, d=64, qbs=64, kbs=64, keep=0.9, causal=False), 1),   # tile lists longer than one chunk
+    (dict(q_lens=[37] * 130, k_lens=[53] * 130, hq=4, hk=2, d=64, qbs=32, kbs=32, keep=0.6, causal=True), 2),           # more sequences than the scheduler holds
+    (dict(q_lens=[128, 70], k_lens=[9000, 4000], hq=4, hk=2, d=64, qbs=64, kbs=128, keep=0.6, causal=True), 2),         # few long items: split over key blocks
+])
+def test_one_launch_form_is_bitwise_the_two_launch_path(spec, launches):
+    """A plain call on 16-bit tensors is one launch whose scheduler reads the sequence boundaries and the
+    mask bytes itself; where that form does not apply the call is pre-pass + attention kernel.  Same tile
+    lists, same kernels body: the results are equal bit for bit, and within tolerance of the oracle."""
+    from hbsattn_amd import set_onepass
+    w = make_problem(seed=96, diag=True, scale=None, **spec)
+    assert _launches(w) == launches
+    out = _run(w)
+    rows = None                                            # the long problems are checked on sampled rows
+    if w.q.shape[0] * w.k.shape[0] * w.q.shape[1] > 2e8:
+        rows = sorted(set(torch.randint(0, w.q.shape[0], (48,), generator=torch.Generator().manual_seed(5)).tolist()
+                          + [0, w.cu_q[1] - 1, w.cu_q[1], w.q.shape[0] - 1]))
+    assert_close_to_oracle(out, oracle_for(w, q_rows=rows), "default path")
+    previous = set_onepass(False)
+    try:
+        assert _launches(w) == 2
+        assert torch.equal(_run(w), out)
+    finally:
+        set_onepass(previous)
+    assert torch.equal(_run(w), out)                       # and again as one launch: the launch record was left at zero
+    if launches == 1:                                      # a mask view whose k block stride is not 1 takes the pre-pass
+        wide = torch.zeros(w.block_mask.shape[0], w.block_mask.shape[1], 2 * w.block_mask.shape[2], dtype=torch.bool, device="cuda")
+        wide[:, :, ::2] = w.block_mask
+        args = list(w.args())
+        args[5] = wide[:, :, ::2]
+        assert torch.equal(HBSAttention(*args), out)
+
+
+def test_one_launch_calls_on_several_streams_do_not_share_a_launch_record():
+    w = make_problem(seed=97, q_lens=[2048, 1024], k_lens=[2048, 3072], hq=16, hk=16, d=128, qbs=128, kbs=128, keep=0.4, diag=True,
+                     causal=True, scale=None)
+    assert _launches(w) == 1
+    ref = _run(w)
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    outs = []
+    for rep in range(3):
+        for st in streams:
+            st.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(st):
+                outs.append(HBSAttention(*w.args()))
+    torch.cuda.synchronize()
+    assert all(torch.equal(o, ref) for o in outs)
 
 
 # ---------------------------------------------------------------------------------------
@@ -586,7 +656,7 @@ def test_a_sequence_that_does_not_fit_the_tensors_is_skipped_not_read_out_of_bou
 
 def test_prepared_masks_are_reused_only_for_unchanged_tensors():
     from hbsattn_amd import interface, set_prepared_cache_size
-    w = make_problem(seed=92, q_lens=[700, 500], k_lens=[700, 900], hq=4, hk=2, d=64, qbs=64, kbs=64, keep=0.4, diag=True,
+    w = make_problem(seed=92, q_lens=[700, 500], k_lens=[700, 900], hq=32, hk=16, d=64, qbs=64, kbs=64, keep=0.4, diag=True,
                      causal=True, scale=None)
     previous = set_prepared_cache_size(4)
     calls = []
@@ -613,9 +683,15 @@ def test_prepared_masks_are_reused_only_for_unchanged_tensors():
         torch.cuda.synchronize()
         assert len(calls) == 4 and torch.equal(short[:700], _run(w)[:700]) and int(short[700:].ne(0).sum()) == 0
         assert len(calls) == 4                                   # ... and the full-length entry is still there
-        set_prepared_cache_size(0)                               # switched off: every call prepares
+        set_prepared_cache_size(0)                               # switched off: a plain call is one launch, no pre-pass
         _run(w), _run(w)
-        assert len(calls) == 6
+        assert len(calls) == 4
+        one = interface.set_onepass(False)                       # ... and without that form every call prepares
+        try:
+            _run(w), _run(w)
+            assert len(calls) == 6
+        finally:
+            interface.set_onepass(one)
     finally:
         interface.hbsa_prepare = real
         set_prepared_cache_size(previous)

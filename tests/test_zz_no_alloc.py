@@ -86,3 +86,50 @@ def test_static_entry_point_refuses_problems_beyond_its_array():
     torch.cuda.synchronize()
     assert rc == -3 and "hbsa_fwd_static holds" in _lib.last_error()
     assert torch.isnan(out.float()).all()
+
+
+def test_static_entry_point_allocates_nothing_and_can_be_captured_into_a_graph():
+    """After a first call (which looks up the array's address and the kernels' launch limits) further calls
+    leave the device's free memory exactly where it was, and a call recorded into a graph (the case the entry
+    point is for: nothing may be allocated under capture) replays to the eager result, every time."""
+    lib = _lib.load()
+    w = make_problem(seed=33, q_lens=[900, 640], k_lens=[1200, 640], hq=8, hk=4, d=128, qbs=64, kbs=128, keep=0.4,
+                     diag=True, causal=True, scale=None)
+    (cu_q, cu_k, qb2b, cu_nqb, cu_nkb), sizes, scale = _common_args(w)
+    out = torch.full_like(w.q, float("nan"))
+    strides = _strides(w, out)
+
+    def call(stream):
+        return lib.hbsa_fwd_static(w.q.data_ptr(), w.k.data_ptr(), w.v.data_ptr(), out.data_ptr(), cu_q.data_ptr(),
+                                   cu_k.data_ptr(), w.block_mask.data_ptr(), qb2b.data_ptr(), cu_nqb.data_ptr(),
+                                   cu_nkb.data_ptr(), _lib.DTYPE_BF16, *sizes, scale, strides, stream)
+
+    main = torch.cuda.current_stream().cuda_stream
+    assert call(main) == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    eager = out.clone()
+    assert torch.equal(eager, _fwd_with_workspace(w))
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        assert call(main) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "hbsa_fwd_static changed the device's free memory"
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        rc = call(side.cuda_stream)
+        graph.capture_end()
+    assert rc == 0, _lib.last_error()
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {replay}"
+        assert call(main) == 0                      # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
