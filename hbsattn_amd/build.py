@@ -15,7 +15,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _ROOT = os.path.dirname(_HERE)
 SOURCES = [os.path.join(_HERE, "csrc", "hbsa_fwd.hip")]
 OUTPUT = os.path.join(_HERE, "libhbsattn_amd.so")
-HAND_ISSUED_READS = "hbsa_fwd_kernel"   # substring of the mangled names of the kernels with hand-issued LDS reads
+HAND_ISSUED_READS = "hbsa_fwd_kernel"   # substring of the mangled names of the kernels with hand-issued LDS reads ...
+COMPILER_ISSUED = "hbsa_fwd_kernelILi256E"   # ... except the head dim 256 instantiations, whose reads the compiler issues
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
 HIPCC_FLAGS = [
@@ -51,7 +52,7 @@ def build(verbose: bool = False) -> str:
     # that kernel spills vector registers is refused.  (The other kernels leave every wait to the
     # compiler; a spill there only costs time and is reported.)
     spills = _vgpr_spills(res.stderr)
-    fatal = {k: v for k, v in spills.items() if HAND_ISSUED_READS in k}
+    fatal = {k: v for k, v in spills.items() if HAND_ISSUED_READS in k and COMPILER_ISSUED not in k}
     if fatal:
         os.remove(OUTPUT)
         raise RuntimeError(f"vector-register spills in {fatal}: reduce register pressure (see the comment here)")

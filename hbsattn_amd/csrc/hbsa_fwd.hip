@@ -287,7 +287,10 @@ __device__ __forceinline__ float half_sum(float x) {
 }
 
 // --------------------------------------------------------------------------------------
-// Main kernel (persistent).  D = head dim (32, 64 or 128); rows of K/V tiles are D*2 bytes.
+// Main kernel (persistent).  D = head dim (32, 64, 128 or 256); rows of K/V tiles are D*2 bytes.  At D = 256 a
+// wavefront's output accumulator and query operand alone are 192 registers, so a CU runs one workgroup of four
+// wavefronts, each with the 512 registers of a SIMD (accumulators in the AGPR half), and its two 128 KB of K/V
+// tile buffers take most of the LDS.
 //
 // Scheduling.  The grid is as many workgroups as fit the device at once and every workgroup
 // loops over work items it claims from eight queues, one per XCD (the chip's eight dies, each
@@ -509,17 +512,28 @@ __device__ __forceinline__ int build_tile_list(int *list, int chunk_base, MoreWo
 // wavefront complete in order, and lds_wait<N> returns once at most N of them are outstanding.
 // (The transposing read is issued this way because the compiler otherwise waits for every
 // outstanding global->LDS load before it; the K reads so that their issue distance is fixed.)
-template <int OFF>
+// HAND = false gives the same reads as ordinary loads the compiler schedules and waits for itself (the
+// lds_wait calls then do nothing): the form for instantiations that spill registers, where a register with
+// a hand-issued read in flight could be saved before its data arrives.
+template <int OFF, bool HAND = true>
 __device__ __forceinline__ short8v lds_read_b128(uint32_t addr) {
-  short8v r;
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(r) : "v"(addr), "n"(OFF));
-  return r;
+  if constexpr (HAND) {
+    short8v r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(r) : "v"(addr), "n"(OFF));
+    return r;
+  } else {
+    return *(const __attribute__((address_space(3))) short8v *)(uintptr_t)(addr + (uint32_t)OFF);
+  }
 }
-template <int OFF>
+template <int OFF, bool HAND = true>
 __device__ __forceinline__ short4v lds_read_tr16_b64(uint32_t addr) {
-  short4v r;
-  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=&v"(r) : "v"(addr), "n"(OFF));
-  return r;
+  if constexpr (HAND) {
+    short4v r;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=&v"(r) : "v"(addr), "n"(OFF));
+    return r;
+  } else {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(uintptr_t)(addr + (uint32_t)OFF));
+  }
 }
 template <int N>
 __device__ __forceinline__ void lds_wait1(short8v &a) {
@@ -544,7 +558,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 }
 
 template <int D, typename E, bool OUT32, int NW, bool EXTRAS, bool FUSED>
-__global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) {
+__global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel(FwdParams p) {
   // OUT32: fp32 output (the fp32-input path; q/k/v are then fp16 staging copies)
   // EXTRAS: the clocked walk, the split over key blocks and the log-sum-exp output are compiled in.  The
   // plain call uses none of them, and its kernel is a tenth shorter without them (1-2 % faster: eight
@@ -563,6 +577,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
   static_assert(LOADS >= 1, "a tile row has fewer 16-byte chunks than the workgroup has wavefronts");
   constexpr int KSTEPS = D / 16;       // MFMA k-steps of Q.K^T
   constexpr int DT = D / 32;           // 32-row tiles of O^T
+  constexpr bool HAND = D <= 128;      // operand reads from LDS issued and waited for by hand (see lds_read_b128)
 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   char *lds_k = lds;
@@ -1185,8 +1200,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
           auto read_k = [&](auto i_) {
             constexpr int i = decltype(i_)::value;
             constexpr int ks = i % KSTEPS;
-            if constexpr (i < KSTEPS) kb[i % PF] = lds_read_b128<0>(k_addr[ks]);
-            else kb[i % PF] = lds_read_b128<32 * RB>(k_addr[ks]);
+            if constexpr (i < KSTEPS) kb[i % PF] = lds_read_b128<0, HAND>(k_addr[ks]);
+            else kb[i % PF] = lds_read_b128<32 * RB, HAND>(k_addr[ks]);
           };
           static_for<0, PF>(read_k);
           // the next tile's K is requested while this tile's first operands are on their way from LDS
@@ -1195,7 +1210,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
           static_for<0, KSTEPS>([&](auto i_) {
             constexpr int i = decltype(i_)::value;
             constexpr int ahead = (NK - 1 - i) < (PF - 1) ? (NK - 1 - i) : (PF - 1);
-            lds_wait1<ahead>(kb[i % PF]);
+            if constexpr (HAND) lds_wait1<ahead>(kb[i % PF]);
             s0 = E::mfma(kb[i % PF], qf[i % KSTEPS], s0);
             if constexpr (i + PF < NK) read_k(std::integral_constant<int, i + PF>{});
           });
@@ -1251,13 +1266,15 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
             constexpr int g = decltype(g_)::value;
             static_for<0, DT>([&](auto dt_) {
               constexpr int dt = decltype(dt_)::value;
-              dst[2 * dt] = lds_read_tr16_b64<g * 16 * RB>(v_addr[dt]);
-              dst[2 * dt + 1] = lds_read_tr16_b64<g * 16 * RB + 8 * RB>(v_addr[dt]);
+              dst[2 * dt] = lds_read_tr16_b64<g * 16 * RB, HAND>(v_addr[dt]);
+              dst[2 * dt + 1] = lds_read_tr16_b64<g * 16 * RB + 8 * RB, HAND>(v_addr[dt]);
             });
           };
           auto wait_vgroup = [&](auto n_, short4v *v) {
             constexpr int n = decltype(n_)::value;
-            if constexpr (DT == 4) {
+            if constexpr (!HAND) {
+              (void)v;   // the compiler waits for its own reads
+            } else if constexpr (DT == 4) {
               lds_wait<n>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]);
             } else if constexpr (DT == 2) {
               asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : "n"(n));
@@ -1280,7 +1297,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void hbsa_fwd_kernel(FwdParams p) 
           static_for<KSTEPS, NK>([&](auto i_) {
             constexpr int i = decltype(i_)::value;
             constexpr int ahead = (NK - 1 - i) < (PF - 1) ? (NK - 1 - i) : (PF - 1);
-            lds_wait1<ahead>(kb[i % PF]);
+            if constexpr (HAND) lds_wait1<ahead>(kb[i % PF]);
             s1 = E::mfma(kb[i % PF], qf[i % KSTEPS], s1);
             if constexpr (i + PF < NK) read_k(std::integral_constant<int, i + PF>{});
           });
@@ -1587,7 +1604,7 @@ inline size_t f32_stage_bytes(int64_t tokens, int64_t heads, int64_t d) { return
 // tensor i (0 q, 1 k, 2 v) of an fp32 call
 F32Tensor f32_tensor(int i, const void *q, const void *k, const void *v, const int64_t *strides, int total_q, int total_k,
                      int nhead_q, int nhead_k, int headdim) {
-  const int dshift = headdim == 32 ? 3 : headdim == 64 ? 4 : 5;
+  const int dshift = headdim == 32 ? 3 : headdim == 64 ? 4 : headdim == 128 ? 5 : 6;
   const void *x = i == 0 ? q : i == 1 ? k : v;
   const int64_t tokens = i == 0 ? total_q : total_k;
   const int heads = i == 0 ? nhead_q : nhead_k;
@@ -1597,7 +1614,9 @@ F32Tensor f32_tensor(int i, const void *q, const void *k, const void *v, const i
 // Wavefronts per workgroup of the 16-bit attention kernel for an item of `slots` wave slots (32-row
 // slices of a q block x q heads of a GQA group): eight when the item has more than four slots, so that
 // one workgroup stages its K/V tiles once (head dims from 64; the fp32 kernel always has four).
-inline int fwd_wavefronts(int slots, int headdim, bool f32_exact) { return (!f32_exact && slots > 4 && headdim >= 64) ? 8 : 4; }
+inline int fwd_wavefronts(int slots, int headdim, bool f32_exact) {
+  return (!f32_exact && slots > 4 && headdim >= 64 && headdim <= 128) ? 8 : 4;
+}
 
 // Split over key blocks pays when the work items cannot fill the device: fewer than one per CU.
 // Returns the number of parts (1 = no split) for the current device.
@@ -1682,7 +1701,7 @@ int launch_fwd_nw(const FwdParams &fp, long long items, hipStream_t stream) {
 template <int D, typename E, bool OUT32>
 int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
   const bool extras = fp.walk != 0 || fp.nparts > 1 || fp.lse != nullptr;
-  if constexpr (D >= 64) {
+  if constexpr (D >= 64 && D <= 128) {
     if (fp.nw == 8)
       return extras ? launch_fwd_nw<D, E, OUT32, 8, true>(fp, items, stream) : launch_fwd_nw<D, E, OUT32, 8, false>(fp, items, stream);
   }
@@ -1691,7 +1710,7 @@ int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
 // the one-launch form (16-bit tensors, none of the extras)
 template <int D, typename E>
 int launch_fwd_fused(const FwdParams &fp, long long items, hipStream_t stream) {
-  if constexpr (D >= 64) {
+  if constexpr (D >= 64 && D <= 128) {
     if (fp.nw == 8) return launch_fwd_nw<D, E, false, 8, false, true>(fp, items, stream);
   }
   return launch_fwd_nw<D, E, false, 4, false, true>(fp, items, stream);
@@ -1715,7 +1734,7 @@ int launch_fwd_fused(const FwdParams &fp, long long items, hipStream_t stream) {
 // LDS: K[64][D+4] and V[64][D+4] floats (the 4-float pad spreads the rows over the banks).
 // --------------------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(kThreads, 2) void hbsa_fwd_f32_kernel(FwdParams p, float c_signed) {
+__global__ __launch_bounds__(kThreads, D > 128 ? 1 : 2) void hbsa_fwd_f32_kernel(FwdParams p, float c_signed) {
   constexpr int LD = D + 4;       // LDS row stride in floats
   constexpr int DJ = D / 8;       // ds_read_b128 steps of S
   constexpr int DT = D / 32;      // 32-row tiles of O^T
@@ -1871,7 +1890,7 @@ int launch_fwd_split(FwdParams &fp, long long items, hipStream_t stream, char *a
   fp.bits = bit_copies;
   int rc = launch_fwd<D, E, OUT32>(fp, items * parts, stream);
   if (rc != 0) return rc;
-  constexpr int dshift = D == 32 ? 3 : D == 64 ? 4 : 5;
+  constexpr int dshift = D == 32 ? 3 : D == 64 ? 4 : D == 128 ? 5 : 6;
   const int64_t n = (int64_t)rows << dshift;
   hipLaunchKernelGGL((hbsa_merge_kernel<E, OUT32>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, fp.part_out,
                      fp.part_lse, final_out, final_lse, fp.sched, parts, total_q, nhead_q, dshift, o_s, o_h, lse_s, lse_h);
@@ -2026,7 +2045,8 @@ int try_onepass(const void *q, const void *k, const void *v, void *out, const in
   switch (headdim) {
     case 32: return bf ? launch_fwd_fused<32, ElemBF16>(fp, items, st) : launch_fwd_fused<32, ElemF16>(fp, items, st);
     case 64: return bf ? launch_fwd_fused<64, ElemBF16>(fp, items, st) : launch_fwd_fused<64, ElemF16>(fp, items, st);
-    default: return bf ? launch_fwd_fused<128, ElemBF16>(fp, items, st) : launch_fwd_fused<128, ElemF16>(fp, items, st);
+    case 128: return bf ? launch_fwd_fused<128, ElemBF16>(fp, items, st) : launch_fwd_fused<128, ElemF16>(fp, items, st);
+    default: return bf ? launch_fwd_fused<256, ElemBF16>(fp, items, st) : launch_fwd_fused<256, ElemF16>(fp, items, st);
   }
 }
 }  // namespace
@@ -2045,7 +2065,7 @@ int hbsa_fwd_launches(int32_t dtype, int32_t batch, int32_t total_k, int32_t nhe
                       int32_t num_q_block, int32_t num_k_block, int32_t q_block_size, int32_t k_block_size,
                       int64_t mask_kblk_stride, void *stream) {
   if (nhead_k <= 0 || nhead_q <= 0 || nhead_q % nhead_k != 0 || num_q_block <= 0 || num_k_block <= 0 || q_block_size <= 0 ||
-      k_block_size <= 0 || (headdim != 32 && headdim != 64 && headdim != 128))
+      k_block_size <= 0 || (headdim != 32 && headdim != 64 && headdim != 128 && headdim != 256))
     return 2;
   const int ratio = nhead_q / nhead_k, wps = (q_block_size + kWaveRows - 1) / kWaveRows;
   const int nw = fwd_wavefronts(ratio * wps, headdim, false);
@@ -2183,8 +2203,8 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
   if (q_block_size <= 0 || k_block_size <= 0 || q_block_size % 16 || k_block_size % 16)
     return fail(HBSA_ERR_INVALID_ARGUMENT, "q_block_size (%d) and k_block_size (%d) must be positive multiples of 16",
                 q_block_size, k_block_size);
-  if (headdim != 32 && headdim != 64 && headdim != 128)
-    return fail(HBSA_ERR_UNSUPPORTED, "headdim %d not in {32, 64, 128}", headdim);
+  if (headdim != 32 && headdim != 64 && headdim != 128 && headdim != 256)
+    return fail(HBSA_ERR_UNSUPPORTED, "headdim %d not in {32, 64, 128, 256}", headdim);
   if (dtype < HBSA_DTYPE_BF16 || dtype > HBSA_DTYPE_F32_STAGED16)
     return fail(HBSA_ERR_UNSUPPORTED, "dtype code %d not supported", dtype);
   if (num_k_block <= 0 || total_k <= 0) return fail(HBSA_ERR_INVALID_ARGUMENT, "no keys");
@@ -2258,7 +2278,8 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
     switch (headdim) {
       case 32: return launch_fwd_f32<32>(fp, c_signed, items, st);
       case 64: return launch_fwd_f32<64>(fp, c_signed, items, st);
-      default: return launch_fwd_f32<128>(fp, c_signed, items, st);
+      case 128: return launch_fwd_f32<128>(fp, c_signed, items, st);
+      default: return launch_fwd_f32<256>(fp, c_signed, items, st);
     }
   }
   if (f32) {
@@ -2274,7 +2295,8 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
     switch (headdim) {
       case 32: return run_fwd<32, ElemF16, true>(fp, items, st, split_area, num_k_block);
       case 64: return run_fwd<64, ElemF16, true>(fp, items, st, split_area, num_k_block);
-      default: return run_fwd<128, ElemF16, true>(fp, items, st, split_area, num_k_block);
+      case 128: return run_fwd<128, ElemF16, true>(fp, items, st, split_area, num_k_block);
+      default: return run_fwd<256, ElemF16, true>(fp, items, st, split_area, num_k_block);
     }
   }
   const bool bf = dtype == HBSA_DTYPE_BF16;
@@ -2283,8 +2305,10 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out, flo
                        : run_fwd<32, ElemF16, false>(fp, items, st, split_area, num_k_block);
     case 64: return bf ? run_fwd<64, ElemBF16, false>(fp, items, st, split_area, num_k_block)
                        : run_fwd<64, ElemF16, false>(fp, items, st, split_area, num_k_block);
-    default: return bf ? run_fwd<128, ElemBF16, false>(fp, items, st, split_area, num_k_block)
-                       : run_fwd<128, ElemF16, false>(fp, items, st, split_area, num_k_block);
+    case 128: return bf ? run_fwd<128, ElemBF16, false>(fp, items, st, split_area, num_k_block)
+                        : run_fwd<128, ElemF16, false>(fp, items, st, split_area, num_k_block);
+    default: return bf ? run_fwd<256, ElemBF16, false>(fp, items, st, split_area, num_k_block)
+                       : run_fwd<256, ElemF16, false>(fp, items, st, split_area, num_k_block);
   }
 }
 
@@ -2305,8 +2329,8 @@ int fwd_call(const void *q, const void *k, const void *v, void *out, const int32
   if (!q || !k || !v || !out) return fail(HBSA_ERR_INVALID_ARGUMENT, "null pointer argument");
   if (nhead_k <= 0 || nhead_q % nhead_k != 0)
     return fail(HBSA_ERR_INVALID_ARGUMENT, "nhead_q (%d) must be divisible by nhead_k (%d)", nhead_q, nhead_k);
-  if (headdim != 32 && headdim != 64 && headdim != 128)
-    return fail(HBSA_ERR_UNSUPPORTED, "headdim %d not in {32, 64, 128}", headdim);
+  if (headdim != 32 && headdim != 64 && headdim != 128 && headdim != 256)
+    return fail(HBSA_ERR_UNSUPPORTED, "headdim %d not in {32, 64, 128, 256}", headdim);
   if (dtype < HBSA_DTYPE_BF16 || dtype > HBSA_DTYPE_F32_STAGED16)
     return fail(HBSA_ERR_UNSUPPORTED, "dtype code %d not supported", dtype);
   if (!std::isfinite(softmax_scale)) return fail(HBSA_ERR_INVALID_ARGUMENT, "softmax_scale is not finite");

@@ -20,7 +20,8 @@ import torch
 from . import _lib
 from .utils import calculate_blocks
 
-_NATIVE_HEADDIMS = (32, 64, 128)
+_NATIVE_HEADDIMS = (32, 64, 128, 256)      # head dims the forward kernels are instantiated for; others run zero-padded
+_BWD_MAX_HEADDIM = 128                      # the backward kernels stop here
 _DTYPE_CODES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16, torch.float32: _lib.DTYPE_F32}
 
 # How fp32 q/k/v are multiplied: "exact" = fp32 matrix instructions, the arithmetic of the reference's
@@ -261,8 +262,8 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = 
 
 def backward_supported(q: torch.Tensor) -> bool:
     """The backward kernels take bf16 / fp16 tensors; head dims up to 128 (others than 32, 64, 128 run
-    zero-padded, like the forward)."""
-    return q.dtype in (torch.bfloat16, torch.float16) and q.dim() == 3 and 0 < q.shape[2] <= _NATIVE_HEADDIMS[-1]
+    zero-padded, like the forward).  The forward alone goes up to head dim 256."""
+    return q.dtype in (torch.bfloat16, torch.float16) and q.dim() == 3 and 0 < q.shape[2] <= _BWD_MAX_HEADDIM
 
 
 def hbsa_backward(q, k, v, out, dout, lse, prepared: PreparedMask, softmax_scale):

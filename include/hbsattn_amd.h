@@ -171,8 +171,11 @@ size_t hbsa_fwd_split_workspace_bytes(int32_t total_q, int32_t nhead_q, int32_t 
  * (process-wide; returns the previous setting; the environment variable HBSATTN_AMD_ONEPASS=0 does the same
  * when the library is loaded).
  *
- * Supported: headdim in {32, 64, 128}; q_block_size, k_block_size positive multiples
- * of 16; nhead_q % nhead_k == 0; every sequence length >= 1.  Query rows with no
+ * Supported: headdim in {32, 64, 128, 256} (the reference pads any head dim to the next power of two,
+ * reference hbsattn/fwd_triton_auto_tile_size.py:269; callers do the same with zero columns up to one of
+ * these); q_block_size, k_block_size positive multiples of 16; nhead_q % nhead_k == 0; every sequence
+ * length >= 1.  At headdim 256 a CU runs one workgroup of four wavefronts whose operand reads the compiler
+ * schedules: it works, at about half the efficiency of the smaller head dims.  Query rows with no
  * visible key produce exactly 0 (reference hbsattn/reference.py:97-98).
  */
 int hbsa_fwd(const void *q, const void *k, const void *v, void *out,

@@ -791,6 +791,47 @@ def test_split_with_many_kv_heads_and_a_head_count_that_is_no_multiple_of_eight(
 
 
 # ---------------------------------------------------------------------------------------
+# head dims above 128 (the reference pads any head dim to a power of two: fwd_triton_auto_tile_size.py:269)
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("d", [160, 192, 256])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_head_dims_up_to_256(d, dtype):
+    from hbsattn_amd import set_fp32_mode, set_onepass
+    specs = [dict(q_lens=[700, 333, 64], k_lens=[900, 333, 200], hq=8, hk=2, qbs=64, kbs=128, keep=0.4, causal=True, scale=None),
+             dict(q_lens=[1024, 2048], k_lens=[1024, 2048], hq=18, hk=18, qbs=128, kbs=128, keep=0.3, causal=False, scale=0.05),
+             dict(q_lens=[300, 512, 77], k_lens=[600, 512, 410], hq=6, hk=3, qbs=80, kbs=48, keep=0.5, causal=True, scale=None)]
+    for n, spec in enumerate(specs):
+        w = make_problem(seed=7000 + n, d=d, diag=True, dtype=dtype, **spec)
+        ref = oracle_for(w)
+        modes = ["exact", "fast"] if dtype == torch.float32 else [None]
+        for mode in modes:
+            previous = set_fp32_mode(mode) if mode else None
+            try:
+                out = _run(w)
+                assert out.shape == w.q.shape and out.dtype == dtype
+                assert_close_to_oracle(out, ref, f"d={d} {dtype} spec {n} {mode}")
+                if dtype != torch.float32:   # ... and through the pre-pass + attention kernel path, bit for bit
+                    one = set_onepass(False)
+                    try:
+                        assert torch.equal(_run(w), out)
+                    finally:
+                        set_onepass(one)
+            finally:
+                if mode:
+                    set_fp32_mode(previous)
+
+
+def test_head_dim_256_log_sum_exp_and_split_over_key_blocks():
+    w = make_problem(seed=7100, q_lens=[128, 70], k_lens=[9000, 4000], hq=4, hk=2, d=256, qbs=64, kbs=128, keep=0.6, diag=True,
+                     causal=True, scale=None)
+    out, lse = _run_lse(w)
+    ref_out, ref_lse = hbsa_oracle(w.q.cpu(), w.k.cpu(), w.v.cpu(), w.cu_q, w.cu_k, w.block_mask.cpu(), w.q_block_size,
+                                   w.k_block_size, w.causal, w.softmax_scale, return_lse=True)
+    assert_close_to_oracle(out, ref_out, "d=256 split")
+    assert (lse.cpu() - ref_lse).abs().max().item() <= 2e-3
+
+
+# ---------------------------------------------------------------------------------------
 # seeded random shapes: lengths, head counts, block sizes, head dims, dtypes, masks
 # ---------------------------------------------------------------------------------------
 def test_seeded_random_shapes_against_the_oracle():
