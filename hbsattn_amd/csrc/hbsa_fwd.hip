@@ -108,6 +108,9 @@ inline FastDiv make_fast_div(uint32_t d) {
   return f;
 }
 
+// (Fields are appended at the end, never inserted: the compiler fetches the kernel arguments in aligned groups,
+// and a layout that splits the fields the tile loop uses makes it fetch some of them again inside that loop,
+// where a scalar load's wait also waits for every hand-issued LDS read; measured, 0.8 % of T for one such shift.)
 struct FwdParams {
   const char *q, *k, *v;
   char *out;
@@ -149,6 +152,7 @@ struct FwdParams {
   const uint8_t *mask;                            // block_mask bytes, innermost (k block) stride 1
   int64_t ms_h, ms_q;                             // its head and q block strides
   int32_t batch, nkb_total, total_k, qbs;
+  int32_t pack;   // host side only: the launch uses the kernel whose wave slots are packed across the q heads of a GQA group
 };
 
 // Boundaries of one sequence of the packed batch, as read from the caller's device arrays.
@@ -557,7 +561,7 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-template <int D, typename E, bool OUT32, int NW, bool EXTRAS, bool FUSED>
+template <int D, typename E, bool OUT32, int NW, bool EXTRAS, bool FUSED, bool PACK>
 __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel(FwdParams p) {
   // OUT32: fp32 output (the fp32-input path; q/k/v are then fp16 staging copies)
   // EXTRAS: the clocked walk, the split over key blocks and the log-sum-exp output are compiled in.  The
@@ -566,6 +570,8 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
   // FUSED: the one-launch form.  No pre-pass has run: wavefront 0 derives an item's geometry from the
   // sequence boundaries (kept in LDS) and its bit row from the item's own block_mask bytes, which it
   // fetches into an LDS staging area one item ahead, where the other form fetches the prepared records.
+  // PACK: wave slots packed across the q heads of a GQA group (see slot_of below); instantiated for the
+  // one-launch form only, since either placement of the queries gives the same results bit for bit.
   // NW: wavefronts (wave slots) of a workgroup, 4 or 8.  Eight are used when the q heads of a GQA group
   // and the 32-row slices of a q block give an item more than four wave slots: one workgroup per CU then
   // stages every K/V tile once for all of them instead of two workgroups staging it each.
@@ -1018,16 +1024,61 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
     }
   };
 
-  // this wave's slice of an item: q head, first row inside the q block, rows
-  auto q_row_ptr = [&](int hk, int sub, int row_begin, int rows, bool &act, int &hq, int &row0, int &nrows) {
+  // This wavefront's slot of an item.  A wave slot holds up to 32 (q head of the GQA group, query row of the
+  // q block) entries.  Plain form: the 32-row slices of one head after another (slot = head * wps + slice), a
+  // q block of 80 rows filling 32 + 32 + 16 entries per head.  Packed form (PACK: q_block_size no multiple
+  // of 32 and several q heads per kv head): entry number = head * rows + row, every slot takes the next 32
+  // numbers, so a slot may hold the last rows of one head and the first rows of the next and only an item's
+  // last slot is partly empty.  Every lane works on one query with its own pointers and causal limit, and
+  // all heads of the group see the same K/V tiles, so nothing else changes.
+  struct Slot {
+    int first;          // first entry number (packed) / first row of the slice (plain)
+    int n;              // entries held, <= 0: none
+    int min_r, max_r;   // smallest and largest query row among them
+    int hq;             // plain form: the slot's q head; packed form: the group's first q head
+  };
+  auto quotient = [](int a, int b) {   // a / b for 0 <= a < 2^20, 0 < b < 2^12
+    return (int)(((float)a + 0.5f) * __builtin_amdgcn_rcpf((float)b));
+  };
+  auto slot_of = [&](int hk, int sub, int rows) -> Slot {
     const int slot = sub * NW + wave;
-    const int head_in_group = slot / p.wps;
-    row0 = (slot % p.wps) * kWaveRows;
-    nrows = min(kWaveRows, rows - row0);
-    act = head_in_group < p.ratio && nrows > 0;
-    hq = hk * p.ratio + head_in_group;
-    const int r = min(row0 + l32, rows - 1);
-    return p.q + (int64_t)(row_begin + r) * p.q_s + (int64_t)hq * p.q_h + g32 * 16;
+    Slot sl;
+    if constexpr (PACK) {
+      sl.hq = hk * p.ratio;
+      sl.first = slot * kWaveRows;
+      sl.n = min(kWaveRows, p.ratio * rows - sl.first);
+      sl.min_r = 0;
+      sl.max_r = rows - 1;
+      if (sl.n > 0) {
+        const int h0 = __builtin_amdgcn_readfirstlane(quotient(sl.first, rows));
+        const int h1 = __builtin_amdgcn_readfirstlane(quotient(sl.first + sl.n - 1, rows));
+        if (h0 == h1) {   // all entries belong to one head
+          sl.min_r = sl.first - h0 * rows;
+          sl.max_r = sl.min_r + sl.n - 1;
+        }
+      }
+    } else {
+      const int head = slot / p.wps;
+      sl.hq = hk * p.ratio + head;
+      sl.first = (slot % p.wps) * kWaveRows;
+      sl.n = head < p.ratio ? min(kWaveRows, rows - sl.first) : 0;
+      sl.min_r = sl.first;
+      sl.max_r = sl.first + sl.n - 1;
+    }
+    return sl;
+  };
+  // q head and row (inside the q block) of entry idx of a slot with entries; idx past the last entry repeats it.
+  // (The plain form needs nothing but the slot: what stays live through an item's tiles is as little as it can be.)
+  auto slot_entry = [&](const Slot &sl, int idx, int rows, int &hq, int &r) {
+    const int e = sl.first + min(idx, sl.n - 1);
+    if constexpr (PACK) {
+      const int h = quotient(e, rows);
+      hq = sl.hq + h;
+      r = e - h * rows;
+    } else {
+      hq = sl.hq;
+      r = e;
+    }
   };
 
   // Q^T fragments (B operand) of one item: lane (l32, g32) ends up with, per k-step ks, the 16 bytes
@@ -1038,15 +1089,15 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
   // (v_permlane16_swap), which leaves k-step 2k in A_k and k-step 2k+1 in B_k.
   short8v qf[KSTEPS];
   auto load_q = [&](int hk, int sub, int row_begin, int rows) {
-    const int slot = sub * NW + wave;
-    const int head_in_group = slot / p.wps;
-    const int row0 = (slot % p.wps) * kWaveRows;
-    if (head_in_group >= p.ratio || rows - row0 <= 0) return;   // this wavefront has no rows: qf is never used
-    const int hq = hk * p.ratio + head_in_group;
-    const char *base = p.q + (int64_t)hq * p.q_h + (lane & 16) * 2 + g32 * 16;
+    const Slot sl = slot_of(hk, sub, rows);
+    if (sl.n <= 0) return;   // this wavefront has no rows: qf is never used
     const int l16 = lane & 15;
-    const char *ra = base + (int64_t)(row_begin + min(row0 + l16, rows - 1)) * p.q_s;
-    const char *rb = base + (int64_t)(row_begin + min(row0 + 16 + l16, rows - 1)) * p.q_s;
+    int hq_a, r_a, hq_b, r_b;
+    slot_entry(sl, l16, rows, hq_a, r_a);
+    slot_entry(sl, 16 + l16, rows, hq_b, r_b);
+    const char *base = p.q + (lane & 16) * 2 + g32 * 16;
+    const char *ra = base + (int64_t)(row_begin + r_a) * p.q_s + (int64_t)hq_a * p.q_h;
+    const char *rb = base + (int64_t)(row_begin + r_b) * p.q_s + (int64_t)hq_b * p.q_h;
     if constexpr (KSTEPS >= 2) {
 #pragma unroll
       for (int k = 0; k < KSTEPS / 2; ++k) {
@@ -1100,8 +1151,20 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
       pending = claim();
     }
 
-    bool active; int hq, row0, nrows;
-    (void)q_row_ptr(cur_hk, cur_sub, row_begin, rows, active, hq, row0, nrows);
+    const Slot slot = slot_of(cur_hk, cur_sub, rows);
+    const int nrows = slot.n;   // lanes l32 < nrows hold a query
+    // last key position this lane's query / any query of the wavefront sees (causal): key position <= q_pos + row + shift
+    int lane_kvis;
+    if constexpr (PACK) {
+      int hq_mine, r_mine = 0;
+      if (nrows > 0) slot_entry(slot, l32, rows, hq_mine, r_mine);
+      lane_kvis = q_pos + r_mine + shift;
+    } else {
+      lane_kvis = q_pos + slot.first + min(l32, nrows - 1) + shift;   // (a wavefront without queries never looks at it)
+    }
+    const int wave_kvis_min = q_pos + slot.min_r + shift;
+    const int wave_kvis_max = q_pos + slot.max_r + shift;
+    const bool active = nrows > 0;
 
     f32x16 o[DT];
 #pragma unroll
@@ -1111,10 +1174,6 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
     float m_run = -INFINITY;  // running reference max, raw (unscaled) score units
     float l_run = 0.f;        // this lane's share of the row sum
 
-    // causal visibility of this lane's / this wave's rows: key position <= qpos + shift
-    const int lane_kvis = q_pos + min(row0 + l32, rows - 1) + shift;
-    const int wave_kvis_min = q_pos + row0 + shift;
-    const int wave_kvis_max = q_pos + row0 + nrows - 1 + shift;
     const char *kg = p.k + (int64_t)cur_hk * p.k_h + (int64_t)key_begin * p.k_s;
     const char *vg = p.v + (int64_t)cur_hk * p.v_h + (int64_t)key_begin * p.v_s;
 
@@ -1396,12 +1455,14 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
 
     // ---- epilogue: normalise, convert, store (rows with no visible key store exact zeros)
     if (active) {
+      int hq, my_r;   // this lane's query (lanes l32 >= nrows repeat the last one and store nothing)
+      slot_entry(slot, l32, rows, hq, my_r);
       const float l_tot = half_sum(l_run);
       const float inv = l_tot > 0.f ? __builtin_amdgcn_rcpf(l_tot) : 0.f;   // 1 ulp; a full division is ten instructions
       if (EXTRAS && p.nparts > 1) {
         // split over key blocks: this part's normalised result and log-sum-exp, for the merge kernel
         if (l32 < nrows) {
-          const int64_t rh = ((int64_t)cur_part * p.total_q + (row_begin + row0 + l32)) * p.nhead_q + hq;
+          const int64_t rh = ((int64_t)cur_part * p.total_q + (row_begin + my_r)) * p.nhead_q + hq;
           if (g32 == 0)
             p.part_lse[rh] = l_tot > 0.f ? (m_run * sm_c + __builtin_amdgcn_logf(l_tot)) * 0.69314718055994531f : -INFINITY;
           float *dst = p.part_out + rh * D;
@@ -1418,11 +1479,11 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
         // natural-log sum over the row's visible keys of exp(scale * q.k); m_run is the (possibly
         // lagging) reference maximum the row sum was accumulated under, which makes this exact
         const float lse = l_tot > 0.f ? (m_run * sm_c + __builtin_amdgcn_logf(l_tot)) * 0.69314718055994531f : -INFINITY;
-        p.lse[(int64_t)(row_begin + row0 + l32) * p.lse_s + (int64_t)hq * p.lse_h] = lse;
+        p.lse[(int64_t)(row_begin + my_r) * p.lse_s + (int64_t)hq * p.lse_h] = lse;
       }
       if constexpr (OUT32) {
         if (l32 < nrows) {
-          char *orow = p.out + (int64_t)(row_begin + row0 + l32) * p.o_s + (int64_t)hq * p.o_h;
+          char *orow = p.out + (int64_t)(row_begin + my_r) * p.o_s + (int64_t)hq * p.o_h;
           const float f = inv * sm_out_mul;
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt)
@@ -1439,8 +1500,12 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
         // lanes i and i+32 (same row) trade halves (16 contiguous bytes per lane), then lanes with
         // bit 4 clear / set (rows l and 16 + l) trade the two 16-dim halves of the block.
         const int l16 = lane & 15;
-        char *row_x = p.out + (int64_t)(row_begin + row0 + l16) * p.o_s + (int64_t)hq * p.o_h + (lane & 16) * 2 + g32 * 16;
-        char *row_y = row_x + (int64_t)16 * p.o_s;
+        int hq_x, r_x, hq_y, r_y;   // the slot's entries l16 and 16 + l16
+        slot_entry(slot, l16, rows, hq_x, r_x);
+        slot_entry(slot, 16 + l16, rows, hq_y, r_y);
+        char *row_x = p.out + (int64_t)(row_begin + r_x) * p.o_s + (int64_t)hq_x * p.o_h + (lane & 16) * 2 + g32 * 16;
+        char *row_y = PACK ? p.out + (int64_t)(row_begin + r_y) * p.o_s + (int64_t)hq_y * p.o_h + (lane & 16) * 2 + g32 * 16
+                           : row_x + (int64_t)16 * p.o_s;   // (a row past the block's end is not stored)
         const bool st_x = l16 < nrows, st_y = 16 + l16 < nrows;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -1611,11 +1676,20 @@ F32Tensor f32_tensor(int i, const void *q, const void *k, const void *v, const i
   return {(const float *)x, strides[2 * i], strides[2 * i + 1], heads, dshift, tokens * heads * headdim / 4};
 }
 
-// Wavefronts per workgroup of the 16-bit attention kernel for an item of `slots` wave slots (32-row
-// slices of a q block x q heads of a GQA group): eight when the item has more than four slots, so that
-// one workgroup stages its K/V tiles once (head dims from 64; the fp32 kernel always has four).
+// Wave slots of an item: 32-row slices of one q head after another, or (the one-launch form, when a q block
+// is no whole number of slices and a kv head serves several q heads) packed across the q heads of the group.
+inline bool fwd_packs(int ratio, int q_block_size) { return ratio > 1 && q_block_size % kWaveRows != 0; }
+inline int fwd_slots(int ratio, int q_block_size, bool packed) {
+  return packed ? (ratio * q_block_size + kWaveRows - 1) / kWaveRows : ratio * ((q_block_size + kWaveRows - 1) / kWaveRows);
+}
+// Wavefronts per workgroup of the 16-bit attention kernel for an item of `slots` wave slots: eight when the
+// item has more than four slots, so that one workgroup stages its K/V tiles once (head dims 64 and 128; the
+// fp32 kernel always has four), unless the item's last workgroup of eight would be at most half full: then
+// workgroups of four, none of them with idle wavefronts (measured at 20 slots, head dim 64: 0.365 -> 0.33 ms).
 inline int fwd_wavefronts(int slots, int headdim, bool f32_exact) {
-  return (!f32_exact && slots > 4 && headdim >= 64 && headdim <= 128) ? 8 : 4;
+  if (f32_exact || slots <= 4 || headdim < 64 || headdim > 128) return 4;
+  const int in_last = slots % 8;
+  return (in_last >= 1 && in_last <= 4) ? 4 : 8;
 }
 
 // Split over key blocks pays when the work items cannot fill the device: fewer than one per CU.
@@ -1657,13 +1731,15 @@ int persistent_grid(const void *kernel, int lds_bytes, int threads) {
 
 // The fields of FwdParams that follow from the call's shape and softmax_scale alone.
 void fill_shape(FwdParams &fp, int nhead_q, int nhead_k, int headdim, int num_q_block, int num_k_block, int q_block_size,
-                int k_block_size, int causal, float softmax_scale, bool f32_exact) {
+                int k_block_size, int causal, float softmax_scale, bool f32_exact, bool may_pack = false) {
   fp.nhead_k = nhead_k;
   fp.nqb = num_q_block; fp.ratio = nhead_q / nhead_k; fp.kbs = k_block_size; fp.wpr = words_per_row(num_k_block);
   fp.causal = causal ? 1 : 0;
   fp.wps = (q_block_size + kWaveRows - 1) / kWaveRows;
-  fp.nw = fwd_wavefronts(fp.ratio * fp.wps, headdim, f32_exact);
-  fp.nsub = (fp.ratio * fp.wps + fp.nw - 1) / fp.nw;
+  fp.pack = may_pack && fwd_packs(fp.ratio, q_block_size) ? 1 : 0;
+  const int slots = fwd_slots(fp.ratio, q_block_size, fp.pack != 0);
+  fp.nw = fwd_wavefronts(slots, headdim, f32_exact);
+  fp.nsub = (slots + fp.nw - 1) / fp.nw;
   fp.div_nsub = make_fast_div((uint32_t)fp.nsub);
   fp.div_nqb = make_fast_div((uint32_t)num_q_block);
   fp.div_kbs = make_fast_div((uint32_t)k_block_size);
@@ -1674,10 +1750,10 @@ void fill_shape(FwdParams &fp, int nhead_q, int nhead_k, int headdim, int num_q_
   fp.lag = kLazyRescaleLog2 / c;
 }
 
-template <int D, typename E, bool OUT32, int NW, bool EXTRAS, bool FUSED = false>
+template <int D, typename E, bool OUT32, int NW, bool EXTRAS, bool FUSED = false, bool PACK = false>
 int launch_fwd_nw(const FwdParams &fp, long long items, hipStream_t stream) {
   constexpr int lds_bytes = 4 * kTileKeys * D * 2 + 2 * H_WORDS * 4 + 2 * kListCap * 4 + (FUSED ? 4 * kSeqCap * 4 + kMaskStage : 0);
-  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS, FUSED>);
+  const void *kernel = reinterpret_cast<const void *>(&hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS, FUSED, PACK>);
   // workgroups that fit the current device at once; the attribute and the occupancy are per device
   static thread_local int resident_of[kMaxDevices] = {};
   int dev = 0;
@@ -1693,7 +1769,7 @@ int launch_fwd_nw(const FwdParams &fp, long long items, hipStream_t stream) {
   const int grid = (int)(items < resident ? items : resident);
   FwdParams launch = fp;
   launch.one_each = items <= resident ? 1 : 0;   // every item gets its own workgroup: no queues, no atomics
-  hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS, FUSED>), dim3(grid), dim3(NW * 64), lds_bytes, stream, launch);
+  hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS, FUSED, PACK>), dim3(grid), dim3(NW * 64), lds_bytes, stream, launch);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail((int)e, "hbsa_fwd_kernel launch: %s", hipGetErrorString(e));
   return 0;
@@ -1711,9 +1787,12 @@ int launch_fwd(const FwdParams &fp, long long items, hipStream_t stream) {
 template <int D, typename E>
 int launch_fwd_fused(const FwdParams &fp, long long items, hipStream_t stream) {
   if constexpr (D >= 64 && D <= 128) {
-    if (fp.nw == 8) return launch_fwd_nw<D, E, false, 8, false, true>(fp, items, stream);
+    if (fp.nw == 8)
+      return fp.pack ? launch_fwd_nw<D, E, false, 8, false, true, true>(fp, items, stream)
+                     : launch_fwd_nw<D, E, false, 8, false, true, false>(fp, items, stream);
   }
-  return launch_fwd_nw<D, E, false, 4, false, true>(fp, items, stream);
+  return fp.pack ? launch_fwd_nw<D, E, false, 4, false, true, true>(fp, items, stream)
+                 : launch_fwd_nw<D, E, false, 4, false, true, false>(fp, items, stream);
 }
 
 
@@ -2026,7 +2105,8 @@ int try_onepass(const void *q, const void *k, const void *v, void *out, const in
                 int32_t k_block_size, int32_t causal, float softmax_scale, const int64_t *strides, hipStream_t st) {
   FwdParams fp;
   std::memset(&fp, 0, sizeof(fp));
-  fill_shape(fp, nhead_q, nhead_k, headdim, num_q_block, num_k_block, q_block_size, k_block_size, causal, softmax_scale, false);
+  fill_shape(fp, nhead_q, nhead_k, headdim, num_q_block, num_k_block, q_block_size, k_block_size, causal, softmax_scale, false,
+             true);
   const long long items = (long long)nhead_k * num_q_block * fp.nsub;
   Sched *sched = onepass_record(dtype, batch, total_k, headdim, num_k_block, k_block_size, strides[10], items, st);
   if (sched == nullptr) return kNotOnePass;
@@ -2067,9 +2147,9 @@ int hbsa_fwd_launches(int32_t dtype, int32_t batch, int32_t total_k, int32_t nhe
   if (nhead_k <= 0 || nhead_q <= 0 || nhead_q % nhead_k != 0 || num_q_block <= 0 || num_k_block <= 0 || q_block_size <= 0 ||
       k_block_size <= 0 || (headdim != 32 && headdim != 64 && headdim != 128 && headdim != 256))
     return 2;
-  const int ratio = nhead_q / nhead_k, wps = (q_block_size + kWaveRows - 1) / kWaveRows;
-  const int nw = fwd_wavefronts(ratio * wps, headdim, false);
-  const long long items = (long long)nhead_k * num_q_block * ((ratio * wps + nw - 1) / nw);
+  const int slots = fwd_slots(nhead_q / nhead_k, q_block_size, fwd_packs(nhead_q / nhead_k, q_block_size));   // as try_onepass
+  const int nw = fwd_wavefronts(slots, headdim, false);
+  const long long items = (long long)nhead_k * num_q_block * ((slots + nw - 1) / nw);
   return onepass_record(dtype, batch, total_k, headdim, num_k_block, k_block_size, mask_kblk_stride, items,
                         (hipStream_t)stream) != nullptr ? 1 : 2;
 }
@@ -2133,9 +2213,9 @@ size_t hbsa_fwd_split_workspace_bytes(int32_t total_q, int32_t nhead_q, int32_t 
                                       int32_t num_q_block, int32_t num_k_block, int32_t q_block_size) {
   if (total_q <= 0 || nhead_q <= 0 || nhead_k <= 0 || headdim <= 0 || num_q_block <= 0 || num_k_block <= 0 || q_block_size <= 0)
     return 0;
-  const int ratio = nhead_q / nhead_k, wps = (q_block_size + kWaveRows - 1) / kWaveRows;
-  const int nw = fwd_wavefronts(ratio * wps, headdim, false);
-  const long long items = (long long)nhead_k * num_q_block * ((ratio * wps + nw - 1) / nw);
+  const int slots = fwd_slots(nhead_q / nhead_k, q_block_size, false);
+  const int nw = fwd_wavefronts(slots, headdim, false);
+  const long long items = (long long)nhead_k * num_q_block * ((slots + nw - 1) / nw);
   return split_bytes(split_parts(items, num_k_block), total_q, nhead_q, nhead_k, headdim, num_q_block, num_k_block);
 }
 
