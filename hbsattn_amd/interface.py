@@ -262,15 +262,27 @@ def hbsa_run(q, k, v, prepared: PreparedMask, softmax_scale, return_lse: bool = 
 
 def backward_supported(q: torch.Tensor) -> bool:
     """The backward kernels take bf16 / fp16 tensors; head dims up to 128 (others than 32, 64, 128 run
-    zero-padded, like the forward).  The forward alone goes up to head dim 256."""
-    return q.dtype in (torch.bfloat16, torch.float16) and q.dim() == 3 and 0 < q.shape[2] <= _BWD_MAX_HEADDIM
+    zero-padded, like the forward).  fp32 tensors get their gradients from the bf16 kernels on rounded
+    copies (``hbsa_backward``).  The forward alone goes up to head dim 256."""
+    return q.dtype in _DTYPE_CODES and q.dim() == 3 and 0 < q.shape[2] <= _BWD_MAX_HEADDIM
 
 
 def hbsa_backward(q, k, v, out, dout, lse, prepared: PreparedMask, softmax_scale):
     """``(dq, dk, dv)`` through ``hbsa_bwd`` on the current stream.  ``out`` and ``lse`` are what
     ``hbsa_run(..., return_lse=True)`` returned for the same q, k, v, prepared mask and scale."""
     if not backward_supported(q):
-        raise NotImplementedError("hbsattn_amd: the backward takes bfloat16 / float16 tensors with headdim <= 128")
+        raise NotImplementedError("hbsattn_amd: the backward takes bfloat16 / float16 / float32 tensors with headdim <= 128")
+    if q.dtype == torch.float32:
+        # There are no fp32 backward kernels (the fp32 matrix rate is a sixteenth of the 16-bit one, and the
+        # backward is 2.5 forwards).  The gradients are those of the bf16 computation on rounded copies of q, k, v
+        # (bf16 keeps fp32's range, so no scaling is involved; 8-bit operand significands, fp32 accumulation): its
+        # forward is run again for the output and log-sum-exp that belong to the rounded operands (the
+        # probabilities the backward forms from them then sum to one), and the gradients are returned as fp32.
+        lo = torch.bfloat16
+        q16, k16, v16 = q.to(lo), k.to(lo), v.to(lo)
+        out16, lse16 = hbsa_run(q16, k16, v16, prepared, softmax_scale, return_lse=True)
+        dq, dk, dv = hbsa_backward(q16, k16, v16, out16, dout.to(lo), lse16, prepared, softmax_scale)
+        return dq.float(), dk.float(), dv.float()
     if prepared.cu_k_seqlens is None:
         raise ValueError("this PreparedMask was built without the sequence boundaries the backward needs")
     _check_on_device(prepared.workspace.device, q=q, k=k, v=v, out=out, dout=dout, lse=lse)
@@ -525,7 +537,7 @@ class _HBSAttentionFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, do):
         # The reference stops here (reference hbsattn/hbsa_interface.py:31-32 raises NotImplementedError);
-        # bf16 / fp16 inputs with a native head dim get their gradients, anything else still raises.
+        # head dims up to 128 get their gradients, anything else still raises.
         if getattr(ctx, "prepared", None) is None:
             raise NotImplementedError("It does not support gradient propagation yet for this dtype / headdim")
         q, k, v, out, lse = ctx.saved_tensors

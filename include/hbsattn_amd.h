@@ -314,6 +314,12 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out,
  *
  * Supported: HBSA_DTYPE_BF16 and HBSA_DTYPE_F16, headdim in {32, 64, 128}.  Every element of dq, dk
  * and dv is written (zeros where no gradient flows); no atomics, so results are deterministic.
+ * There are no fp32 backward kernels: the fp32 matrix rate is a sixteenth of the 16-bit one and a backward
+ * is 2.5 forwards of matrix work.  A caller with fp32 tensors passes bf16 copies of q, k, v, out and dout
+ * (bf16 keeps fp32's range), with out and lse from a forward on those copies, and widens the gradients, which
+ * is what the Python operator does.
+ * Head dims above 128 are refused: the dK/dV kernel keeps K^T or V^T of a wavefront's keys and one accumulator
+ * in registers, 241 of 256 at headdim 128.
  */
 size_t hbsa_bwd_workspace_bytes(int32_t total_q, int32_t nhead_q);
 

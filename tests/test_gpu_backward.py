@@ -166,9 +166,30 @@ def test_strided_tensors_give_the_gradients_of_their_contiguous_copies(d):
     _check(got[2], rdv, "dv")
 
 
-def test_float32_inputs_still_raise_like_the_reference():
+@pytest.mark.parametrize("fp32_mode", ["exact", "fast"])
+def test_float32_inputs_get_gradients_of_bf16_accuracy(fp32_mode):
+    """fp32 q, k, v: the forward runs in the chosen fp32 mode, the gradients come from the bf16 kernels on
+    rounded copies with the forward's log-sum-exp, returned as fp32, within the 16-bit tolerance of the oracle."""
+    from hbsattn_amd import HBSAttention, set_fp32_mode
+    previous = set_fp32_mode(fp32_mode)
+    try:
+        for n, (q_lens, k_lens, hq, hk, d, qbs, kbs, causal) in enumerate([([300, 64], [400, 64], 4, 2, 64, 48, 80, True),
+                                                                          ([512], [512], 2, 2, 128, 128, 128, False),
+                                                                          ([130, 70], [130, 90], 4, 2, 18, 32, 16, True)]):
+            q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(140 + n, q_lens, k_lens, hq, hk, d, qbs, kbs, 0.6, torch.float32)
+            out, dq, dk, dv = _gpu_grads(q, k, v, do, cq, ck, mask, qbs, kbs, causal, None)
+            assert dq.dtype == dk.dtype == dv.dtype == torch.float32
+            rdq, rdk, rdv = hbsa_oracle_grads(q, k, v, do, cu_q, cu_k, mask, qbs, kbs, causal, None)
+            _check(dq, rdq, f"fp32 {fp32_mode} case {n} dq")
+            _check(dk, rdk, f"fp32 {fp32_mode} case {n} dk")
+            _check(dv, rdv, f"fp32 {fp32_mode} case {n} dv")
+    finally:
+        set_fp32_mode(previous)
+
+
+def test_head_dims_above_128_still_raise_in_the_backward_like_the_reference():
     from hbsattn_amd import HBSAttention
-    q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(14, [64], [64], 2, 2, 32, 32, 32, 1.1, torch.float32)
+    q, k, v, do, cu_q, cu_k, cq, ck, mask = _problem(14, [64], [64], 2, 2, 160, 32, 32, 1.1, torch.bfloat16)
     qd = q.cuda().requires_grad_(True)
     out = HBSAttention(qd, k.cuda(), v.cuda(), cq, ck, mask.cuda(), 32, 32, False, None)
     with pytest.raises(NotImplementedError):

@@ -790,6 +790,41 @@ def test_split_with_many_kv_heads_and_a_head_count_that_is_no_multiple_of_eight(
     assert (lse.cpu() - ref_lse).abs().max().item() <= 2e-3
 
 
+def test_seeded_random_shapes_that_fill_the_device_as_one_launch_and_as_two():
+    """Random shapes with enough (kv head, q block) items to run unsplit, so that the one-launch path (wave
+    slots packed across the q heads of a group where a q block is no whole number of 32-row slices) and the
+    pre-pass + attention kernel path (plain slots) can be compared bit for bit, both against the oracle."""
+    import random
+    from hbsattn_amd import set_onepass
+    rng = random.Random(777)
+    ones = 0
+    for case in range(24):
+        batch = rng.randint(1, 5)
+        q_lens = [rng.randint(200, 1500) for _ in range(batch)]
+        k_lens = q_lens if rng.random() < 0.4 else [rng.randint(100, 2000) for _ in range(batch)]
+        hk = rng.choice([8, 12, 16, 24])
+        ratio = rng.choice([1, 2, 3, 4])
+        d = rng.choice([32, 64, 128, 128, 256])
+        qbs = 16 * rng.randint(1, 7)
+        kbs = 16 * rng.randint(1, 10)
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        causal = rng.random() < 0.6
+        w = make_problem(seed=9500 + case, q_lens=q_lens, k_lens=k_lens, hq=hk * ratio, hk=hk, d=d, qbs=qbs, kbs=kbs,
+                         keep=rng.choice([0.1, 0.4, 0.9]), diag=True, causal=causal, scale=None, dtype=dtype)
+        what = f"case {case}: q={q_lens} k={k_lens} heads={hk * ratio}/{hk} d={d} blocks={qbs}x{kbs} {dtype} causal={causal}"
+        ones += _launches(w) == 1
+        out = _run(w)
+        rows = sorted(set(torch.randint(0, w.q.shape[0], (64,), generator=torch.Generator().manual_seed(case)).tolist()
+                          + [0, w.q.shape[0] - 1]))
+        assert_close_to_oracle(out, oracle_for(w, q_rows=rows), what)
+        previous = set_onepass(False)
+        try:
+            assert torch.equal(_run(w), out), what
+        finally:
+            set_onepass(previous)
+    assert ones >= 20
+
+
 # ---------------------------------------------------------------------------------------
 # head dims above 128 (the reference pads any head dim to a power of two: fwd_triton_auto_tile_size.py:269)
 # ---------------------------------------------------------------------------------------
@@ -847,7 +882,7 @@ def test_seeded_random_shapes_against_the_oracle():
             k_lens = q_lens if same else [rng.randint(1, 900) for _ in range(batch)]
             hk = rng.choice([1, 2, 3, 5, 9])
             ratio = rng.choice([1, 1, 2, 4, 7])
-            d = rng.choice([16, 24, 32, 40, 64, 72, 96, 128])
+            d = rng.choice([16, 24, 32, 40, 64, 72, 96, 128, 144, 200, 256])
             qbs = 16 * rng.randint(1, 12)
             kbs = 16 * rng.randint(1, 12)
             dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
