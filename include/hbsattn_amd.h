@@ -217,7 +217,9 @@ int hbsa_fwd_v(const void *const *ptrs, size_t workspace_bytes, const int32_t *s
  * array: calls on one stream are ordered and safe; calls that overlap on one GPU (different streams
  * or host threads) race on it and must be serialised by the caller.  The first call on a device looks
  * up the array's address and the kernels' launch limits (host-side queries, no allocation): make it
- * before a stream capture begins, not inside one.
+ * before a stream capture begins, not inside one.  The call always runs as pre-pass + attention kernel on
+ * the array (never as hbsa_fwd's one-launch form, whose launch record belongs to a stream), so it can be
+ * recorded into a graph and the graph replayed on any stream.
  */
 #define HBSA_STATIC_SCRATCH_BYTES (32u << 20)
 int hbsa_fwd_static(const void *q, const void *k, const void *v, void *out,
