@@ -175,7 +175,7 @@ size_t hbsa_fwd_split_workspace_bytes(int32_t total_q, int32_t nhead_q, int32_t 
  * reference hbsattn/fwd_triton_auto_tile_size.py:269; callers do the same with zero columns up to one of
  * these); q_block_size, k_block_size positive multiples of 16; nhead_q % nhead_k == 0; every sequence
  * length >= 1.  At headdim 256 a CU runs one workgroup of four wavefronts whose operand reads the compiler
- * schedules: it works, at about half the efficiency of the smaller head dims.  Query rows with no
+ * schedules: it works, at about two thirds of the efficiency of headdim 128.  Query rows with no
  * visible key produce exactly 0 (reference hbsattn/reference.py:97-98).
  */
 int hbsa_fwd(const void *q, const void *k, const void *v, void *out,
