@@ -83,7 +83,11 @@ def _call_fwd(lib, **over):
 ])
 def test_argument_validation_reports_errors_without_touching_the_gpu(over, code, needle):
     lib = _lib.load()
-    rc = _call_fwd(lib, **over)
+    one = lib.hbsa_set_onepass(0)   # (on a machine with a GPU the one-launch form would need no workspace and launch)
+    try:
+        rc = _call_fwd(lib, **over)
+    finally:
+        lib.hbsa_set_onepass(one)
     assert rc == code
     assert needle in _lib.last_error()
 
@@ -183,3 +187,39 @@ def test_host_calculate_blocks_rejects_bad_input():
     small = np.zeros(3, dtype=np.int32)
     assert lib.hbsa_calculate_blocks(cu.ctypes.data, 1, 16, ctypes.addressof(nb), None, small.ctypes.data, None, 2) == -3
     assert nb.value == 7
+
+
+def test_array_form_entry_point_validates_like_hbsa_fwd():
+    """hbsa_fwd_v is hbsa_fwd with its arguments in arrays: same checks, same codes, nothing launched."""
+    lib = _lib.load()
+    fwd_v = lib.hbsa_fwd_v_locked
+    strides = (ctypes.c_int64 * 11)(4096, 128, 4096, 128, 4096, 128, 4096, 128, 1, 1, 1)
+    ptrs = (ctypes.c_void_p * 11)(*([256] * 11))
+    sizes = (ctypes.c_int32 * 12)(0, 1, 128, 128, 30, 4, 128, 1, 1, 128, 128, 1)          # 30 q heads on 4 kv heads
+    a = lambda x: ctypes.addressof(x)
+    assert fwd_v(a(ptrs), 1 << 30, a(sizes), 0.1, a(strides), None) == -1 and "divisible" in _lib.last_error()
+    sizes[4] = 32; sizes[5] = 32; sizes[6] = 96                                            # head dim 96
+    assert fwd_v(a(ptrs), 1 << 30, a(sizes), 0.1, a(strides), None) == -2 and "headdim" in _lib.last_error()
+    sizes[6] = 128; sizes[2] = 0                                                           # no queries: nothing to do
+    assert fwd_v(a(ptrs), 1 << 30, a(sizes), 0.1, a(strides), None) == 0
+    assert fwd_v(None, 0, a(sizes), 0.1, a(strides), None) == -1 and "null" in _lib.last_error()
+
+
+def test_a_call_without_a_device_reports_two_launches_and_asks_for_its_workspace():
+    """Whether a call runs as one launch is a host-side question (sizes, strides, the stream's state); without a
+    device to run on the answer is the two-launch form, and hbsa_fwd without a workspace is refused, not launched."""
+    lib = _lib.load()
+    args = (_lib.DTYPE_BF16, 8, 65536, 32, 32, 128, 512, 512, 128, 128, 1, None)
+    assert lib.hbsa_fwd_launches(*args) in (1, 2)                       # 2 here (no GPU), 1 on an MI355X
+    assert lib.hbsa_fwd_launches(_lib.DTYPE_F32, *args[1:]) == 2        # fp32 tensors never run as one launch
+    assert lib.hbsa_fwd_launches(_lib.DTYPE_BF16, 200, *args[2:]) == 2  # nor do more than 127 sequences
+    assert lib.hbsa_fwd_launches(*args[:10], 2, None) == 2              # nor a mask whose k block stride is not 1
+    previous = lib.hbsa_set_onepass(0)
+    try:
+        assert lib.hbsa_fwd_launches(*args) == 2
+        assert lib.hbsa_set_onepass(1) == 0
+    finally:
+        lib.hbsa_set_onepass(previous)
+    import torch
+    if not torch.cuda.is_available():
+        assert _call_fwd(lib, ws=None, ws_bytes=0) == -3 and "workspace" in _lib.last_error()
