@@ -27,7 +27,10 @@
 // two buffers (three for the Q tiles of the D = 128 dK/dV kernel): tile t + 1 travels while tile t is computed
 // on, one barrier per tile.  A tile that is
 // read both by rows and transposed is stored once, in a layout without bank conflicts for either
-// (BwdTile::swz_both).  The forward's persistent scheduling is not applied here.
+// (BwdTile::swz_both).  In the dQ kernel and the D = 128 dK/dV kernel the operand reads from LDS are issued by
+// hand, a fixed number ahead of the products that use them (BwdOperandOffsets).  The forward's persistent
+// scheduling is not applied here: the grids already start their heaviest workgroups first, and what bounds
+// both kernels at long sequences is the stream of tiles from memory next to the matrix work, not the tail.
 
 namespace {
 
@@ -73,6 +76,61 @@ struct BwdTile {
 // 16 bytes per lane from global memory (scalar base + 32-bit lane offset) straight into LDS at lds_addr + 16 * lane
 __device__ __forceinline__ void bwd_dma16(uint32_t lds_addr, const char *sbase, uint32_t voff) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+
+// ---- Operand reads issued by hand (lds_read_b128 / lds_read_tr16_b64 of the forward, which explain the rules):
+// the compiler puts a read next to the product that uses it, and a chain of products on one accumulator then
+// waits out the LDS latency at every step.  Here a fixed number of reads is under way ahead of the products.
+//
+// Per-lane byte offsets of the operands inside a tile stored with BwdTile::swz_both, computed once per kernel:
+//   rows[ks]   : row lane % 32 (+ 32 * h as an immediate), the 16 bytes of step ks for this lane's half of the step
+//   tr[dt]     : the first of the two transposing reads of head dim slice dt for keys 16 * g .. (+ g * 16 rows as an
+//                immediate); the second one, eight rows further down, sits at (tr[dt] ^ 32) + 8 rows: for every
+//                head dim swz_both(key + 8) = swz_both(key) ^ 2 when key < 8
+template <int D>
+struct BwdOperandOffsets {
+  using T = BwdTile<D>;
+  uint32_t rows[T::KSTEPS], tr[T::DT];
+  __device__ __forceinline__ void init(int lane) {
+    const int l32 = lane & 31, g32 = lane >> 5;
+    const int rd = l32 * T::RB + ((g32 ^ T::swz_both(l32)) << 4);
+#pragma unroll
+    for (int ks = 0; ks < T::KSTEPS; ++ks) rows[ks] = (uint32_t)(rd ^ (ks * 32));
+    const int key = 4 * g32 + ((lane & 15) >> 2);
+    const int lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+    const int t0 = key * T::RB + ((lc ^ T::swz_both(key)) << 4) + 8 * (lane & 1);
+#pragma unroll
+    for (int dt = 0; dt < T::DT; ++dt) tr[dt] = (uint32_t)(t0 ^ (dt * 64));
+  }
+};
+
+// the 2 * DT transposing reads of key group G of the tile at LDS address tile (all head dim slices)
+template <int D, int G>
+__device__ __forceinline__ void bwd_issue_transposed(const BwdOperandOffsets<D> &off, uint32_t tile, short4v *dst) {
+  using T = BwdTile<D>;
+  static_for<0, T::DT>([&](auto dt_) {
+    constexpr int dt = decltype(dt_)::value;
+    dst[2 * dt] = lds_read_tr16_b64<G * 16 * T::RB>(off.tr[dt] + tile);
+    dst[2 * dt + 1] = lds_read_tr16_b64<G * 16 * T::RB + 8 * T::RB>((off.tr[dt] ^ 32u) + tile);
+  });
+}
+// returns once at most N LDS operations issued after those 2 * DT reads are outstanding
+template <int D, int N>
+__device__ __forceinline__ void bwd_wait_transposed(short4v *v) {
+  constexpr int DT = BwdTile<D>::DT;
+  static_assert(N <= 15, "the counter has four bits");
+  if constexpr (DT == 4) lds_wait<N>(v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]);
+  else if constexpr (DT == 2) asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : "n"(N));
+  else asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(v[0]), "+v"(v[1]) : "n"(N));
+}
+// acc[dt] += (those operands)^T . packed
+template <int D, typename E>
+__device__ __forceinline__ void bwd_transposed_products(const short4v *v, short8v packed, f32x16 *acc) {
+#pragma unroll
+  for (int dt = 0; dt < BwdTile<D>::DT; ++dt) {
+    const short8v va = __builtin_shufflevector(v[2 * dt], v[2 * dt + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+    acc[dt] = E::mfma(va, packed, acc[dt]);
+  }
 }
 
 // rows 32*h .. 32*h+31 of the tile . frag^T, the forward's S^T = K Q^T for one half of a tile
@@ -231,6 +289,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
     for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
 
   const int lane_kvis = inf.q_pos + min(row0 + l32, inf.rows - 1) + inf.shift;   // last key position the row sees (causal)
+  const int wave_kvis_min = inf.q_pos + min(row0, inf.rows - 1) + inf.shift;      // ... the wavefront's first row sees
   const uint32_t *bits = p.bits + ((size_t)hk * p.nqb + qb) * p.wpr;
   const char *kg = p.k + (int64_t)hk * p.k_h + (int64_t)inf.key_begin * p.k_s;
   const char *vg = p.v + (int64_t)hk * p.v_h + (int64_t)inf.key_begin * p.v_s;
@@ -274,6 +333,12 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
       bwd_dma16(dst + (uint32_t)(T::TILE_BYTES + i * 4 * 1024), vsrc, rr * v_s32 + ld_chunk);
     }
   };
+  BwdOperandOffsets<D> off;
+  off.init(lane);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)HBSA_AS3(lds);
+  // Reads of one half tile's two chains S^T = K Q^T and dP^T = V dO^T: K and V rows in turn, PF under way
+  constexpr int PF = 3, NC = 2 * T::KSTEPS;
+  static_assert(NC >= PF, "the first reads of a half are issued as one group");
   bool have = next_tile();
   int buf = 0;
   if (have) fetch(0);
@@ -281,7 +346,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
     const int cur_kpos = kpos, valid = tile_valid();
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the tile has landed
     __syncthreads();                      // ... every wavefront's, and the other buffer has been read by all
-    const char *k_t = lds + buf * 2 * T::TILE_BYTES, *v_t = k_t + T::TILE_BYTES;
+    const uint32_t k_t = lds_base + (uint32_t)(buf * 2 * T::TILE_BYTES), v_t = k_t + (uint32_t)T::TILE_BYTES;
     have = next_tile();
     if (have) fetch(buf ^ 1);   // on its way while this tile is computed on
     buf ^= 1;
@@ -289,22 +354,58 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
     int lim = valid;   // keys of the tile below lim are visible to this lane's row
     if (p.causal) lim = min(lim, lane_kvis - cur_kpos + 1);
     lim -= 4 * g32;
+    short8v rb[PF];
+    auto chain_read = [&](auto h_, auto i_) {
+      constexpr int h = decltype(h_)::value, i = decltype(i_)::value;
+      rb[i % PF] = lds_read_b128<h * 32 * T::RB>(off.rows[i >> 1] + ((i & 1) ? v_t : k_t));
+    };
+    // edge: some key of the tile is hidden from some row of the wavefront (the tile's end, or the causal
+    // diagonal); elsewhere the per-element comparison and select are left out.  Rows past the block's end
+    // have lse2 = +inf and so P = 0 either way.
+    const bool edge = valid < kTileKeys || (p.causal && cur_kpos + valid - 1 > wave_kvis_min);
+    auto half = [&](auto h_) {
+      constexpr int h = decltype(h_)::value;
+      f32x16 s, dp;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const f32x16 s = bwd_rows_times_frag<D, E>(k_t, h, qf, lane);
-      const f32x16 dp = bwd_rows_times_frag<D, E>(v_t, h, dof, lane);
-      float e[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const bool vis = 32 * h + 8 * (i >> 2) + (i & 3) < lim;
-        const float pv = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], p.c, -lse2)) : 0.f;
-        e[i] = pv * (dp[i] - dlt);
-      }
+      for (int i = 0; i < 16; ++i) { s[i] = 0.f; dp[i] = 0.f; }
+      static_for<0, NC>([&](auto i_) {
+        constexpr int i = decltype(i_)::value;
+        constexpr int ahead = (NC - 1 - i) < (PF - 1) ? (NC - 1 - i) : (PF - 1);
+        lds_wait1<ahead>(rb[i % PF]);
+        if constexpr (i & 1) dp = E::mfma(rb[i % PF], dof[i >> 1], dp);
+        else s = E::mfma(rb[i % PF], qf[i >> 1], s);
+        if constexpr (i + PF < NC) chain_read(h_, std::integral_constant<int, i + PF>{});
+      });
+      // The K^T operands of this half's first dQ products are on their way while the vector ALU forms dS, and
+      // behind them (first half) the first reads of the second half's chains.
+      short4v tb[2][2 * T::DT];
+      bwd_issue_transposed<D, 2 * h>(off, k_t, tb[0]);
+      if constexpr (h == 0)
+        static_for<0, PF>([&](auto i_) { chain_read(std::integral_constant<int, 1>{}, i_); });
       short8v lo, hi;
-      bwd_pack<E>(e, lo, hi);
-      bwd_transposed_times_packed<D, E>(k_t, 2 * h, lo, lane, acc);
-      bwd_transposed_times_packed<D, E>(k_t, 2 * h + 1, hi, lane, acc);
-    }
+      auto form_ds = [&](auto edge_) {
+        float e[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i], p.c, -lse2));
+          if constexpr (decltype(edge_)::value) pv = 32 * h + 8 * (i >> 2) + (i & 3) < lim ? pv : 0.f;
+          e[i] = pv * (dp[i] - dlt);
+        }
+        bwd_pack<E>(e, lo, hi);
+      };
+      if (edge) form_ds(std::true_type{});
+      else form_ds(std::false_type{});
+      // the second key group's operands travel during the first group's products (the registers for both
+      // at once, next to dS in the making, are not there)
+      bwd_issue_transposed<D, 2 * h + 1>(off, k_t, tb[1]);
+      bwd_wait_transposed<D, 2 * T::DT + (h == 0 ? PF : 0)>(tb[0]);
+      bwd_transposed_products<D, E>(tb[0], lo, acc);
+      bwd_wait_transposed<D, 0>(tb[1]);
+      bwd_transposed_products<D, E>(tb[1], hi, acc);
+    };
+    static_for<0, PF>([&](auto i_) { chain_read(std::integral_constant<int, 0>{}, i_); });
+    half(std::integral_constant<int, 0>{});
+    half(std::integral_constant<int, 1>{});
   }
   if (active && l32 < nrows)
     bwd_store_rows<D, E>(p.dq + (int64_t)(inf.row_begin + row0 + l32) * p.dq_s + (int64_t)hq * p.dq_h, acc, p.scale, g32);
@@ -576,6 +677,7 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   const bool active = nrows > 0;
   const int key_pos = kbl * p.kbs + min(row0 + l32, krows - 1);
   const int wg_first_key = kbl * p.kbs + wg_row0;
+  const int wave_key_max = kbl * p.kbs + min(row0 + kWaveRows - 1, krows - 1);   // position of the wavefront's last key
 
   // this wavefront's resident operand: K^T (P wavefront) or V^T (dS wavefront) of its 32 keys; lane holds
   // key l32, d = 16 * ks + 8 * g32 .. + 7
@@ -670,6 +772,9 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   // this lane's 4 x 16 bytes of a (tile parity, slot, half) record of P
   char *p_mine = p_buf + (size_t)slot * 8192 + lane * 16;
 
+  BwdOperandOffsets<D> off;
+  off.init(lane);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)HBSA_AS3(lds);   // Q tiles at 0, 1, 2 tile sizes, dO tiles at 3, 4
   // The loop exists once per role (the same barriers in both): with the roles as branches of one loop body the
   // register allocator keeps both roles' temporaries apart and spills.
   auto run = [&](auto role_) {
@@ -698,40 +803,83 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
       if (cur) fetch(q_after, par ^ 1);   // on its way during this iteration (the buffers it fills were last read an iteration ago)
     }
     if (active) {
+      // Operand reads are issued by hand (BwdOperandOffsets): PF reads of a pair of chains under way ahead of
+      // their products, the transposing reads of a key group before the vector ALU work that precedes their
+      // products.  The counts in the waits name only reads that every path issues.
+      constexpr int PF = 4, NC = 2 * T::KSTEPS;
+      short8v rb[PF];
+      short4v tb[2][2 * T::DT];
       if constexpr (ROLE == 0) {
         if (had) {   // ---- P wavefront, current tile
-          const char *q_t = q_buf + q_now * T::TILE_BYTES, *g_t = g_buf + par * T::TILE_BYTES;
+          const uint32_t q_t = lds_base + (uint32_t)(q_now * T::TILE_BYTES), g_t = lds_base + (uint32_t)((3 + par) * T::TILE_BYTES);
           int first_vis = 0;   // rows of the tile from first_vis on see this lane's key (causal)
           if (p.causal) first_vis = max(0, key_pos - shift - first_q_pos);
           if (l32 >= nrows) first_vis = 64;
+          // S = Q K^T of both halves of the tile, their steps in turn (read i: half i % 2, step i / 2)
+          auto chain_read = [&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            rb[i % PF] = lds_read_b128<(i & 1) * 32 * T::RB>(off.rows[i >> 1] + q_t);
+          };
+          static_for<0, PF>(chain_read);
+          f32x16 sv[2];
 #pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const f32x16 sv = bwd_rows_times_frag<D, E>(q_t, h, frag, lane);
+          for (int i = 0; i < 16; ++i) { sv[0][i] = 0.f; sv[1][i] = 0.f; }
+          static_for<0, NC>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            constexpr int ahead = (NC - 1 - i) < (PF - 1) ? (NC - 1 - i) : (PF - 1);
+            lds_wait1<ahead>(rb[i % PF]);
+            sv[i & 1] = E::mfma(rb[i % PF], frag[i >> 1], sv[i & 1]);
+            if constexpr (i + PF < NC) chain_read(std::integral_constant<int, i + PF>{});
+          });
+          bwd_issue_transposed<D, 0>(off, g_t, tb[0]);
+          bwd_issue_transposed<D, 1>(off, g_t, tb[1]);
+          // edge: some row of the tile does not see some key of the wavefront (the causal diagonal, or a slot
+          // with fewer than 32 keys); elsewhere the per-element comparison and select are left out.
+          const bool edge = nrows < kWaveRows || (p.causal && wave_key_max - shift - first_q_pos > 0);
+          auto half = [&](auto h_) {
+            constexpr int h = decltype(h_)::value;
             float ep[16];
+            auto form_p = [&](auto edge_) {
 #pragma unroll
-            for (int a = 0; a < 4; ++a) {
-              const int rr0 = 32 * h + 8 * a + 4 * g32;
-              const f32x4 l4 = *(const f32x4 *)(lse_s + par * 64 + rr0);
+              for (int a = 0; a < 4; ++a) {
+                const int rr0 = 32 * h + 8 * a + 4 * g32;
+                const f32x4 l4 = *(const f32x4 *)(lse_s + par * 64 + rr0);
 #pragma unroll
-              for (int bq = 0; bq < 4; ++bq) {
-                const bool vis = rr0 + bq >= first_vis;   // rows past the block's end carry lse = +inf, hence P = 0
-                ep[4 * a + bq] = vis ? __builtin_amdgcn_exp2f(__builtin_fmaf(sv[4 * a + bq], p.c, -l4[bq])) : 0.f;
+                for (int bq = 0; bq < 4; ++bq) {
+                  float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[h][4 * a + bq], p.c, -l4[bq]));   // rows past the block's end carry lse = +inf, hence P = 0
+                  if constexpr (decltype(edge_)::value) pv = rr0 + bq >= first_vis ? pv : 0.f;
+                  ep[4 * a + bq] = pv;
+                }
               }
-            }
+            };
+            if (edge) form_p(std::true_type{});
+            else form_p(std::false_type{});
 #pragma unroll
             for (int a = 0; a < 4; ++a)
               *(f32x4 *)(p_mine + par * 32768 + h * 4096 + a * 1024) = f32x4{ep[4 * a], ep[4 * a + 1], ep[4 * a + 2], ep[4 * a + 3]};
             short8v plo, phi;
             bwd_pack<E>(ep, plo, phi);
-            bwd_transposed_times_packed<D, E>(g_t, 2 * h, plo, lane, acc);
-            bwd_transposed_times_packed<D, E>(g_t, 2 * h + 1, phi, lane, acc);
-          }
+            bwd_wait_transposed<D, 2 * T::DT>(tb[0]);
+            bwd_transposed_products<D, E>(tb[0], plo, acc);
+            if constexpr (h == 0) bwd_issue_transposed<D, 2>(off, g_t, tb[0]);
+            bwd_wait_transposed<D, (h == 0 ? 2 * T::DT : 0)>(tb[1]);
+            bwd_transposed_products<D, E>(tb[1], phi, acc);
+            if constexpr (h == 0) bwd_issue_transposed<D, 3>(off, g_t, tb[1]);
+          };
+          half(std::integral_constant<int, 0>{});
+          half(std::integral_constant<int, 1>{});
         }
       } else {
+        const uint32_t q_t = lds_base + (uint32_t)(q_before * T::TILE_BYTES), g_t = lds_base + (uint32_t)((3 + par) * T::TILE_BYTES);
+        auto chain_read = [&](auto i_) {   // dP = dO V^T of both halves of the current tile, as above
+          constexpr int i = decltype(i_)::value;
+          rb[i % PF] = lds_read_b128<(i & 1) * 32 * T::RB>(off.rows[i >> 1] + g_t);
+        };
         if (prev) {   // ---- dS wavefront, the tile before: dS = P * (dP - delta), dK^T += Q^T dS
-          const char *q_t = q_buf + q_before * T::TILE_BYTES;
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
+          bwd_issue_transposed<D, 0>(off, q_t, tb[0]);
+          bwd_issue_transposed<D, 1>(off, q_t, tb[1]);
+          auto half = [&](auto h_) {
+            constexpr int h = decltype(h_)::value;
             float ed[16];
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
@@ -743,14 +891,27 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
             }
             short8v dlo, dhi;
             bwd_pack<E>(ed, dlo, dhi);
-            bwd_transposed_times_packed<D, E>(q_t, 2 * h, dlo, lane, acc);
-            bwd_transposed_times_packed<D, E>(q_t, 2 * h + 1, dhi, lane, acc);
-          }
+            bwd_wait_transposed<D, 2 * T::DT>(tb[0]);
+            bwd_transposed_products<D, E>(tb[0], dlo, acc);
+            if constexpr (h == 0) bwd_issue_transposed<D, 2>(off, q_t, tb[0]);
+            bwd_wait_transposed<D, (h == 0 ? 2 * T::DT : 0)>(tb[1]);
+            bwd_transposed_products<D, E>(tb[1], dhi, acc);
+            if constexpr (h == 0) bwd_issue_transposed<D, 3>(off, q_t, tb[1]);
+          };
+          half(std::integral_constant<int, 0>{});
+          half(std::integral_constant<int, 1>{});
         }
         if (had) {   // ---- dS wavefront, current tile: dP = dO V^T, kept for the next iteration
-          const char *g_t = g_buf + par * T::TILE_BYTES;
+          static_for<0, PF>(chain_read);
 #pragma unroll
-          for (int h = 0; h < 2; ++h) dp_prev[h] = bwd_rows_times_frag<D, E>(g_t, h, frag, lane);
+          for (int i = 0; i < 16; ++i) { dp_prev[0][i] = 0.f; dp_prev[1][i] = 0.f; }
+          static_for<0, NC>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            constexpr int ahead = (NC - 1 - i) < (PF - 1) ? (NC - 1 - i) : (PF - 1);
+            lds_wait1<ahead>(rb[i % PF]);
+            dp_prev[i & 1] = E::mfma(rb[i % PF], frag[i >> 1], dp_prev[i & 1]);
+            if constexpr (i + PF < NC) chain_read(std::integral_constant<int, i + PF>{});
+          });
         }
       }
     }
