@@ -24,8 +24,8 @@
 //                           S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS.
 // Both recompute S.  The kept blocks of a mask row or column are found with one load per 32 or 64
 // blocks, not one per block.  Tiles go from global memory straight into LDS (global_load_lds_dwordx4),
-// two buffers (three for the Q tiles of the D = 128 dK/dV kernel): tile t + 1 travels while tile t is computed
-// on, one barrier per tile.  A tile that is
+// two buffers: tile t + 1 travels while tile t is computed on, one barrier per tile (the D = 128 dK/dV kernel
+// has four Q and three dO buffers and fetches two tiles ahead).  A tile that is
 // read both by rows and transposed is stored once, in a layout without bank conflicts for either
 // (BwdTile::swz_both).  In the dQ kernel and the D = 128 dK/dV kernel the operand reads from LDS are issued by
 // hand, a fixed number ahead of the products that use them (BwdOperandOffsets).  The forward's persistent
@@ -39,6 +39,7 @@ struct BwdParams {
   char *dq, *dk, *dv;
   const float *lse;           // [total_q, nhead_q], contiguous
   float *delta;               // [total_q, nhead_q], contiguous: rowsum(dO * O), written by the dQ kernel, read by the dK/dV kernels
+  float *lse2;                // [total_q, nhead_q]: lse * log2(e), +inf where lse is -inf; written by the dQ kernel for the D = 128 dK/dV kernel
   const QBlockInfo *info;
   const uint32_t *bits;
   const int32_t *cu_k, *cu_num_q_block, *cu_num_k_block;
@@ -76,6 +77,11 @@ struct BwdTile {
 // 16 bytes per lane from global memory (scalar base + 32-bit lane offset) straight into LDS at lds_addr + 16 * lane
 __device__ __forceinline__ void bwd_dma16(uint32_t lds_addr, const char *sbase, uint32_t voff) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+
+// 4 bytes per lane likewise, to lds_addr + 4 * lane
+__device__ __forceinline__ void bwd_dma4(uint32_t lds_addr, const void *sbase, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
 }
 
 // ---- Operand reads issued by hand (lds_read_b128 / lds_read_tr16_b64 of the forward, which explain the rules):
@@ -277,7 +283,10 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
       }
     }
     dlt = half_sum(dlt);
-    if (g32 == 0 && l32 < nrows) p.delta[(int64_t)my_row * p.nhead_q + hq] = dlt;
+    if (g32 == 0 && l32 < nrows) {
+      p.delta[(int64_t)my_row * p.nhead_q + hq] = dlt;
+      p.lse2[(int64_t)my_row * p.nhead_q + hq] = lse2;
+    }
   } else {
 #pragma unroll
     for (int ks = 0; ks < T::KSTEPS; ++ks) { qf[ks] = short8v{0, 0, 0, 0, 0, 0, 0, 0}; dof[ks] = qf[ks]; }
@@ -321,23 +330,41 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   const int ld_row = RPL * wave + lane / T::CPR;                                  // + 4 * RPL * i
   const uint32_t ld_chunk = (uint32_t)(((lane % T::CPR) ^ T::swz_both(ld_row)) * 16);
   const uint32_t k_s32 = (uint32_t)p.k_s, v_s32 = (uint32_t)p.v_s;              // the host checks that they fit
+  const uint32_t k_voff = (uint32_t)ld_row * k_s32 + ld_chunk, v_voff = (uint32_t)ld_row * v_s32 + ld_chunk;   // of a full tile's first load
   const uint32_t tiles_addr = (uint32_t)(uintptr_t)HBSA_AS3(lds) + (uint32_t)wave * 1024u;
   auto fetch = [&](int buf) {   // the tile next_tile() has just moved to
     const int valid = tile_valid();
     const char *ksrc = kg + (int64_t)kpos * p.k_s, *vsrc = vg + (int64_t)kpos * p.v_s;
     const uint32_t dst = tiles_addr + (uint32_t)(buf * 2 * T::TILE_BYTES);
+    if (valid == kTileKeys) {   // a full tile: the loads differ in their scalar base only
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-      const uint32_t rr = (uint32_t)min(ld_row + 4 * RPL * i, valid - 1);   // rows past the end repeat the last one (masked later)
-      bwd_dma16(dst + (uint32_t)(i * 4 * 1024), ksrc, rr * k_s32 + ld_chunk);
-      bwd_dma16(dst + (uint32_t)(T::TILE_BYTES + i * 4 * 1024), vsrc, rr * v_s32 + ld_chunk);
+      for (int i = 0; i < LOADS; ++i) {
+        bwd_dma16(dst + (uint32_t)(i * 4 * 1024), ksrc + (int64_t)(4 * RPL * i) * p.k_s, k_voff);
+        bwd_dma16(dst + (uint32_t)(T::TILE_BYTES + i * 4 * 1024), vsrc + (int64_t)(4 * RPL * i) * p.v_s, v_voff);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < LOADS; ++i) {
+        const uint32_t rr = (uint32_t)min(ld_row + 4 * RPL * i, valid - 1);   // rows past the end repeat the last one (masked later)
+        bwd_dma16(dst + (uint32_t)(i * 4 * 1024), ksrc, rr * k_s32 + ld_chunk);
+        bwd_dma16(dst + (uint32_t)(T::TILE_BYTES + i * 4 * 1024), vsrc, rr * v_s32 + ld_chunk);
+      }
     }
   };
+  // Operand addresses of the K tile in use (the V tile lies one tile further, an immediate): they move to the
+  // other buffer with one addition per tile instead of one per read.
   BwdOperandOffsets<D> off;
   off.init(lane);
-  const uint32_t lds_base = (uint32_t)(uintptr_t)HBSA_AS3(lds);
+  {
+    const uint32_t lds_base = (uint32_t)(uintptr_t)HBSA_AS3(lds);
+#pragma unroll
+    for (int ks = 0; ks < T::KSTEPS; ++ks) off.rows[ks] += lds_base;
+#pragma unroll
+    for (int dt = 0; dt < T::DT; ++dt) off.tr[dt] += lds_base;   // a multiple of 64: the second read's "^ 32" still holds
+  }
+  int off_buf = 0;   // the buffer they point to
   // Reads of one half tile's two chains S^T = K Q^T and dP^T = V dO^T: K and V rows in turn, PF under way
-  constexpr int PF = 3, NC = 2 * T::KSTEPS;
+  constexpr int PF = 4, NC = 2 * T::KSTEPS;
   static_assert(NC >= PF, "the first reads of a half are issued as one group");
   bool have = next_tile();
   int buf = 0;
@@ -346,18 +373,26 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
     const int cur_kpos = kpos, valid = tile_valid();
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the tile has landed
     __syncthreads();                      // ... every wavefront's, and the other buffer has been read by all
-    const uint32_t k_t = lds_base + (uint32_t)(buf * 2 * T::TILE_BYTES), v_t = k_t + (uint32_t)T::TILE_BYTES;
+    const int cur_buf = buf;
     have = next_tile();
     if (have) fetch(buf ^ 1);   // on its way while this tile is computed on
     buf ^= 1;
     if (!active) continue;
+    if (off_buf != cur_buf) {
+      const uint32_t step = (uint32_t)((cur_buf - off_buf) * 2 * T::TILE_BYTES);
+#pragma unroll
+      for (int ks = 0; ks < T::KSTEPS; ++ks) off.rows[ks] += step;
+#pragma unroll
+      for (int dt = 0; dt < T::DT; ++dt) off.tr[dt] += step;
+      off_buf = cur_buf;
+    }
     int lim = valid;   // keys of the tile below lim are visible to this lane's row
     if (p.causal) lim = min(lim, lane_kvis - cur_kpos + 1);
     lim -= 4 * g32;
     short8v rb[PF];
     auto chain_read = [&](auto h_, auto i_) {
       constexpr int h = decltype(h_)::value, i = decltype(i_)::value;
-      rb[i % PF] = lds_read_b128<h * 32 * T::RB>(off.rows[i >> 1] + ((i & 1) ? v_t : k_t));
+      rb[i % PF] = lds_read_b128<h * 32 * T::RB + (i & 1) * T::TILE_BYTES>(off.rows[i >> 1]);
     };
     // edge: some key of the tile is hidden from some row of the wavefront (the tile's end, or the causal
     // diagonal); elsewhere the per-element comparison and select are left out.  Rows past the block's end
@@ -379,7 +414,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
       // The K^T operands of this half's first dQ products are on their way while the vector ALU forms dS, and
       // behind them (first half) the first reads of the second half's chains.
       short4v tb[2][2 * T::DT];
-      bwd_issue_transposed<D, 2 * h>(off, k_t, tb[0]);
+      bwd_issue_transposed<D, 2 * h>(off, 0u, tb[0]);
       if constexpr (h == 0)
         static_for<0, PF>([&](auto i_) { chain_read(std::integral_constant<int, 1>{}, i_); });
       short8v lo, hi;
@@ -397,7 +432,7 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
       else form_ds(std::false_type{});
       // the second key group's operands travel during the first group's products (the registers for both
       // at once, next to dS in the making, are not there)
-      bwd_issue_transposed<D, 2 * h + 1>(off, k_t, tb[1]);
+      bwd_issue_transposed<D, 2 * h + 1>(off, 0u, tb[1]);
       bwd_wait_transposed<D, 2 * T::DT + (h == 0 ? PF : 0)>(tb[0]);
       bwd_transposed_products<D, E>(tb[0], lo, acc);
       bwd_wait_transposed<D, 0>(tb[1]);
@@ -634,20 +669,23 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dkv_kernel(BwdParams p) 
 // products between them, each with one operand and one accumulator in registers:
 //   the P wavefront  keeps K^T:  S = Q K^T,  P = exp(S - lse) (masked),   dV^T += dO^T P,   hands P over;
 //   the dS wavefront keeps V^T:  dP = dO V^T,  dS = P * (dP - delta),      dK^T += Q^T dS.
-// P travels through LDS in fp32 (8 KB per slot and tile; dS is formed from the unrounded P), and one tile late: in the iteration in which the P wavefront works on tile t, the dS wavefront
+// P travels through LDS in the element type, as the P wavefront packs it for its own product (4 KB per slot and
+// tile), and one tile late: in the iteration in which the P wavefront works on tile t, the dS wavefront
 // finishes tile t - 1 (whose dP it kept in registers) and forms dP of tile t, so one barrier per tile orders
-// everything.  Hence three Q tile buffers (tile t - 1 is still read while tile t + 1 arrives), two for dO.
-// Tiles go from global memory straight into LDS, stored once in the layout of BwdTile::swz_both.
+// everything.  Tiles go from global memory straight into LDS, stored once in the layout of BwdTile::swz_both,
+// and two tiles ahead (one workgroup per CU has nobody else to cover its waits for memory): four Q buffers
+// (tile t - 1 is still read while tile t + 2 arrives), three for dO, and with them three and four sets of the
+// rows' log-sum-exp and delta, which wavefront 0 loads into LDS the same way.
 template <typename E>
 __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   constexpr int D = 128;
   using T = BwdTile<D>;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  char *q_buf = lds;                                   // [3] Q tiles
-  char *g_buf = lds + 3 * T::TILE_BYTES;               // [2] dO tiles
-  char *p_buf = lds + 5 * T::TILE_BYTES;               // [2 tile parities][4 slots][2 halves][4][64 lanes] four floats
-  float *lse_s = (float *)(lds + 9 * T::TILE_BYTES);   // [2][64] log2-domain log-sum-exp of the tile's rows
-  float *dlt_s = lse_s + 128;                          // [3][64] their delta
+  char *q_buf = lds;                                   // [4] Q tiles
+  char *g_buf = lds + 4 * T::TILE_BYTES;               // [3] dO tiles
+  char *p_buf = lds + 7 * T::TILE_BYTES;               // [2 tile parities][4 slots][2 halves][2][64 lanes] eight 16-bit values
+  float *lse_s = (float *)(lds + 9 * T::TILE_BYTES);   // [3][64] log2-domain log-sum-exp of the tile's rows (index: the dO buffer's)
+  float *dlt_s = lse_s + 192;                          // [4][64] their delta (index: the Q buffer's)
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -748,59 +786,92 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
   const uint32_t q_s32 = (uint32_t)p.q_s, do_s32 = (uint32_t)p.do_s;      // the host checks that they fit
   const uint32_t q_addr = (uint32_t)(uintptr_t)HBSA_AS3(q_buf) + (uint32_t)wave * 1024u;
   const uint32_t g_addr = (uint32_t)(uintptr_t)HBSA_AS3(g_buf) + (uint32_t)wave * 1024u;
-  float l2_next = INFINITY, dl_next = 0.f;
+  const uint32_t q_voff = (uint32_t)ld_row * q_s32 + ld_chunk, g_voff = (uint32_t)ld_row * do_s32 + ld_chunk;   // of a full tile's first load
+  const uint32_t row_addr = (uint32_t)(uintptr_t)HBSA_AS3(lse_s);
+  // Loads of one tile per wavefront: two Q and two dO loads, and in wavefront 0 the two loads of the rows' values
   auto fetch = [&](int qi, int gi) {   // the tile next_tile() has moved to, into Q buffer qi and dO buffer gi
     const int valid = min(64, inf.rows - qoff);
     const int64_t row_first = inf.row_begin + qoff;
     const int hq = hk * p.ratio + r;
     const char *qsrc = p.q + row_first * p.q_s + (int64_t)hq * p.q_h;
     const char *gsrc = p.dout + row_first * p.do_s + (int64_t)hq * p.do_h;
+    if (valid == 64) {   // a full tile: the loads differ in their scalar base only
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const uint32_t rr = (uint32_t)min(ld_row + 32 * i, valid - 1);   // rows past the block's end repeat its last row
-      bwd_dma16(q_addr + (uint32_t)(qi * T::TILE_BYTES + i * 8 * 1024), qsrc, rr * q_s32 + ld_chunk);
-      bwd_dma16(g_addr + (uint32_t)(gi * T::TILE_BYTES + i * 8 * 1024), gsrc, rr * do_s32 + ld_chunk);
+      for (int i = 0; i < 2; ++i) {
+        bwd_dma16(q_addr + (uint32_t)(qi * T::TILE_BYTES + i * 8 * 1024), qsrc + (int64_t)(32 * i) * p.q_s, q_voff);
+        bwd_dma16(g_addr + (uint32_t)(gi * T::TILE_BYTES + i * 8 * 1024), gsrc + (int64_t)(32 * i) * p.do_s, g_voff);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const uint32_t rr = (uint32_t)min(ld_row + 32 * i, valid - 1);   // rows past the block's end repeat its last row
+        bwd_dma16(q_addr + (uint32_t)(qi * T::TILE_BYTES + i * 8 * 1024), qsrc, rr * q_s32 + ld_chunk);
+        bwd_dma16(g_addr + (uint32_t)(gi * T::TILE_BYTES + i * 8 * 1024), gsrc, rr * do_s32 + ld_chunk);
+      }
     }
-    l2_next = INFINITY;   // rows past the block's end take no part: P = exp2(-inf) = 0
-    dl_next = 0.f;
-    if (threadIdx.x < valid) {
-      const float l = p.lse[(row_first + threadIdx.x) * p.nhead_q + hq];
-      l2_next = l == -INFINITY ? INFINITY : l * kLog2e;
-      dl_next = p.delta[(row_first + threadIdx.x) * p.nhead_q + hq];
+    if (wave == 0) {   // the rows' log-sum-exp and delta, one row per lane (rows past the block's end repeat its last row)
+      const uint32_t rvoff = (uint32_t)min(lane, valid - 1) * (uint32_t)(p.nhead_q * 4);
+      bwd_dma4(row_addr + (uint32_t)(gi * 256), p.lse2 + row_first * p.nhead_q + hq, rvoff);
+      bwd_dma4(row_addr + (uint32_t)(768 + qi * 256), p.delta + row_first * p.nhead_q + hq, rvoff);
     }
   };
-  // this lane's 4 x 16 bytes of a (tile parity, slot, half) record of P
-  char *p_mine = p_buf + (size_t)slot * 8192 + lane * 16;
+  // this lane's 2 x 16 bytes of a (tile parity, slot, half) record of P
+  char *p_mine = p_buf + (size_t)slot * 4096 + lane * 16;
 
   BwdOperandOffsets<D> off;
   off.init(lane);
-  const uint32_t lds_base = (uint32_t)(uintptr_t)HBSA_AS3(lds);   // Q tiles at 0, 1, 2 tile sizes, dO tiles at 3, 4
+  const uint32_t lds_base = (uint32_t)(uintptr_t)HBSA_AS3(lds);   // Q tiles at 0 .. 3 tile sizes, dO tiles at 4 .. 6
   // The loop exists once per role (the same barriers in both): with the roles as branches of one loop body the
   // register allocator keeps both roles' temporaries apart and spills.
   auto run = [&](auto role_) {
   constexpr int ROLE = decltype(role_)::value;
-  bool cur = next_tile();   // a tile for this iteration
-  bool prev = false;        // the tile before it exists: its dK part is still due
-  int qi = 0, par = 0;      // Q buffer (of three) and parity of the current tile
+  // Tiles are fetched two ahead: tile t lives in Q buffer t % 4 and dO buffer t % 3 (the dS wavefront still reads
+  // Q of tile t - 1 in the iteration in which tile t + 2 arrives).
+  int n_ahead = 0;                               // tiles fetched and not computed on yet
+  int qi_f = 0, gi_f = 0;                        // buffers of the next fetch
+  int fq_a = 0, fq_b = 0, va_a = 64, va_b = 64;  // first query position and row count of those tiles (a: the older)
+  // Everything loaded so far (the resident operand above all) has arrived before the first tile is requested: the
+  // compiler counts only the loads it knows, and a wait of its own for them inside the loop would also wait for
+  // every tile under way.
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+  bool more = next_tile();
+  auto issue = [&]() {   // fetches the tile next_tile() stands on and moves on
+    const int fq = inf.q_pos + qoff, va = min(64, inf.rows - qoff);
+    if (n_ahead == 0) { fq_a = fq; va_a = va; } else { fq_b = fq; va_b = va; }
+    fetch(qi_f, gi_f);
+    qi_f = (qi_f + 1) & 3;
+    gi_f = gi_f == 2 ? 0 : gi_f + 1;
+    ++n_ahead;
+    more = next_tile();
+  };
+  if (more) issue();
+  if (more) issue();
+  bool prev = false;        // the tile before the current one exists: its dK part is still due
+  int qi = 0, gi = 0, par = 0;   // Q buffer, dO buffer and parity of the current tile
   f32x16 dp_prev[2];        // dS wavefront: dP of the previous tile, both halves
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
     for (int i = 0; i < 16; ++i) dp_prev[h][i] = 0.f;
-  if (cur) fetch(0, 0);
-  while (cur || prev) {
-    const int first_q_pos = inf.q_pos + qoff, shift = inf.shift;   // of the current tile (if any)
-    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the current tile has landed (and its lse, delta)
-    if (cur && threadIdx.x < 64) {
-      lse_s[par * 64 + threadIdx.x] = l2_next;
-      dlt_s[qi * 64 + threadIdx.x] = dl_next;
+  const int shift = inf.shift;
+  while (n_ahead > 0 || prev) {
+    const bool had = n_ahead > 0;
+    const int first_q_pos = fq_a, valid = va_a;   // of the current tile (if any)
+    // This wavefront's part of the current tile has landed; the loads of the tile after it (a wavefront's loads
+    // return in order) may still be under way.
+    if (n_ahead >= 2) {
+      if (wave == 0) __builtin_amdgcn_s_waitcnt(0x0F76);   // vmcnt(6)
+      else __builtin_amdgcn_s_waitcnt(0x0F74);             // vmcnt(4)
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
     }
     __syncthreads();   // ... every wavefront's; what the iteration before read and wrote is settled
-    const int q_now = qi, q_before = qi == 0 ? 2 : qi - 1, q_after = qi == 2 ? 0 : qi + 1;
-    const bool had = cur;
-    if (cur) {
-      cur = next_tile();
-      if (cur) fetch(q_after, par ^ 1);   // on its way during this iteration (the buffers it fills were last read an iteration ago)
+    const int q_now = qi, q_before = (qi + 3) & 3;
+    if (had) {
+      fq_a = fq_b;
+      va_a = va_b;
+      --n_ahead;
+      if (more) issue();   // two tiles ahead: the buffers it fills were last read an iteration ago
     }
     if (active) {
       // Operand reads are issued by hand (BwdOperandOffsets): PF reads of a pair of chains under way ahead of
@@ -811,7 +882,7 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
       short4v tb[2][2 * T::DT];
       if constexpr (ROLE == 0) {
         if (had) {   // ---- P wavefront, current tile
-          const uint32_t q_t = lds_base + (uint32_t)(q_now * T::TILE_BYTES), g_t = lds_base + (uint32_t)((3 + par) * T::TILE_BYTES);
+          const uint32_t q_t = lds_base + (uint32_t)(q_now * T::TILE_BYTES), g_t = lds_base + (uint32_t)((4 + gi) * T::TILE_BYTES);
           int first_vis = 0;   // rows of the tile from first_vis on see this lane's key (causal)
           if (p.causal) first_vis = max(0, key_pos - shift - first_q_pos);
           if (l32 >= nrows) first_vis = 64;
@@ -833,9 +904,10 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
           });
           bwd_issue_transposed<D, 0>(off, g_t, tb[0]);
           bwd_issue_transposed<D, 1>(off, g_t, tb[1]);
-          // edge: some row of the tile does not see some key of the wavefront (the causal diagonal, or a slot
-          // with fewer than 32 keys); elsewhere the per-element comparison and select are left out.
-          const bool edge = nrows < kWaveRows || (p.causal && wave_key_max - shift - first_q_pos > 0);
+          // edge: some row of the tile does not see some key of the wavefront (the causal diagonal, a slot with
+          // fewer than 32 keys, a tile with fewer than 64 rows); elsewhere the per-element comparison and select
+          // are left out.
+          const bool edge = nrows < kWaveRows || valid < 64 || (p.causal && wave_key_max - shift - first_q_pos > 0);
           auto half = [&](auto h_) {
             constexpr int h = decltype(h_)::value;
             float ep[16];
@@ -843,22 +915,21 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
 #pragma unroll
               for (int a = 0; a < 4; ++a) {
                 const int rr0 = 32 * h + 8 * a + 4 * g32;
-                const f32x4 l4 = *(const f32x4 *)(lse_s + par * 64 + rr0);
+                const f32x4 l4 = *(const f32x4 *)(lse_s + gi * 64 + rr0);
 #pragma unroll
                 for (int bq = 0; bq < 4; ++bq) {
-                  float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[h][4 * a + bq], p.c, -l4[bq]));   // rows past the block's end carry lse = +inf, hence P = 0
-                  if constexpr (decltype(edge_)::value) pv = rr0 + bq >= first_vis ? pv : 0.f;
+                  float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[h][4 * a + bq], p.c, -l4[bq]));
+                  if constexpr (decltype(edge_)::value) pv = (rr0 + bq >= first_vis && rr0 + bq < valid) ? pv : 0.f;   // rows past the block's end repeat its last row
                   ep[4 * a + bq] = pv;
                 }
               }
             };
             if (edge) form_p(std::true_type{});
             else form_p(std::false_type{});
-#pragma unroll
-            for (int a = 0; a < 4; ++a)
-              *(f32x4 *)(p_mine + par * 32768 + h * 4096 + a * 1024) = f32x4{ep[4 * a], ep[4 * a + 1], ep[4 * a + 2], ep[4 * a + 3]};
             short8v plo, phi;
             bwd_pack<E>(ep, plo, phi);
+            *(short8v *)(p_mine + par * 16384 + h * 2048) = plo;
+            *(short8v *)(p_mine + par * 16384 + h * 2048 + 1024) = phi;
             bwd_wait_transposed<D, 2 * T::DT>(tb[0]);
             bwd_transposed_products<D, E>(tb[0], plo, acc);
             if constexpr (h == 0) bwd_issue_transposed<D, 2>(off, g_t, tb[0]);
@@ -870,7 +941,7 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
           half(std::integral_constant<int, 1>{});
         }
       } else {
-        const uint32_t q_t = lds_base + (uint32_t)(q_before * T::TILE_BYTES), g_t = lds_base + (uint32_t)((3 + par) * T::TILE_BYTES);
+        const uint32_t q_t = lds_base + (uint32_t)(q_before * T::TILE_BYTES), g_t = lds_base + (uint32_t)((4 + gi) * T::TILE_BYTES);
         auto chain_read = [&](auto i_) {   // dP = dO V^T of both halves of the current tile, as above
           constexpr int i = decltype(i_)::value;
           rb[i % PF] = lds_read_b128<(i & 1) * 32 * T::RB>(off.rows[i >> 1] + g_t);
@@ -881,13 +952,18 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
           auto half = [&](auto h_) {
             constexpr int h = decltype(h_)::value;
             float ed[16];
+            const u32x4 pw[2] = {*(const u32x4 *)(p_mine + (par ^ 1) * 16384 + h * 2048),
+                                 *(const u32x4 *)(p_mine + (par ^ 1) * 16384 + h * 2048 + 1024)};
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
               const int rr0 = 32 * h + 8 * a + 4 * g32;
               const f32x4 d4 = *(const f32x4 *)(dlt_s + q_before * 64 + rr0);
-              const f32x4 p4 = *(const f32x4 *)(p_mine + (par ^ 1) * 32768 + h * 4096 + a * 1024);
 #pragma unroll
-              for (int bq = 0; bq < 4; ++bq) ed[4 * a + bq] = p4[bq] * (dp_prev[h][4 * a + bq] - d4[bq]);
+              for (int bq = 0; bq < 4; ++bq) {
+                const uint32_t w = pw[a >> 1][2 * (a & 1) + (bq >> 1)];
+                const float pv = (bq & 1) ? E::hi(w) : E::lo(w);
+                ed[4 * a + bq] = pv * (dp_prev[h][4 * a + bq] - d4[bq]);
+              }
             }
             short8v dlo, dhi;
             bwd_pack<E>(ed, dlo, dhi);
@@ -916,7 +992,8 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
       }
     }
     prev = had;
-    qi = q_after;
+    qi = (qi + 1) & 3;
+    gi = gi == 2 ? 0 : gi + 1;
     par ^= 1;
   }
   if (active && l32 < nrows) {

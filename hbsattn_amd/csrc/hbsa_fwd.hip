@@ -2502,7 +2502,7 @@ int hbsa_fwd_static(const void *q, const void *k, const void *v, void *out, cons
 
 size_t hbsa_bwd_workspace_bytes(int32_t total_q, int32_t nhead_q) {
   if (total_q < 0 || nhead_q < 0) return 0;
-  return align_up((size_t)total_q * nhead_q * sizeof(float), 256);
+  return 2 * align_up((size_t)total_q * nhead_q * sizeof(float), 256);   // delta and the scaled log-sum-exp of every (row, q head)
 }
 
 int hbsa_bwd(const void *q, const void *k, const void *v, const void *out, const void *dout, const float *lse, void *dq,
@@ -2551,6 +2551,7 @@ int hbsa_bwd(const void *q, const void *k, const void *v, const void *out, const
   bp.q = (const char *)q; bp.k = (const char *)k; bp.v = (const char *)v; bp.out = (const char *)out; bp.dout = (const char *)dout;
   bp.dq = (char *)dq; bp.dk = (char *)dk; bp.dv = (char *)dv;
   bp.lse = lse; bp.delta = (float *)bwd_workspace;
+  bp.lse2 = bp.delta + align_up((size_t)total_q * nhead_q * sizeof(float), 256) / sizeof(float);
   bp.info = (const QBlockInfo *)workspace;
   bp.bits = (const uint32_t *)((const char *)workspace + bits_offset(nhead_k, num_q_block));
   bp.cu_k = cu_k_seqlens; bp.cu_num_q_block = cu_num_q_block; bp.cu_num_k_block = cu_num_k_block;

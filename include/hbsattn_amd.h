@@ -311,6 +311,7 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out,
  *   workspace   as left by hbsa_fwd_prepare (or hbsa_fwd) for the same mask, sequence boundaries,
  *               block sizes and `causal`; read only
  *   bwd_workspace  >= hbsa_bwd_workspace_bytes(total_q, nhead_q) bytes of device scratch, 16-byte aligned
+ *               (two floats per (row, q head): rowsum(dout * out) and the scaled log-sum-exp)
  *   strides     int64[16] = { q_tok, q_head, k_tok, k_head, v_tok, v_head, out_tok, out_head,
  *                             dout_tok, dout_head, dq_tok, dq_head, dk_tok, dk_head, dv_tok, dv_head }
  *

@@ -134,7 +134,7 @@ def test_backward_argument_validation_without_touching_the_gpu(over, code, needl
 
 def test_backward_workspace_bytes_and_empty_problem():
     lib = _lib.load()
-    assert lib.hbsa_bwd_workspace_bytes(100, 8) == 3328      # 100 * 8 floats, rounded up to 256 bytes
+    assert lib.hbsa_bwd_workspace_bytes(100, 8) == 2 * 3328  # two arrays of 100 * 8 floats, each rounded up to 256 bytes
     assert lib.hbsa_bwd_workspace_bytes(0, 8) == 0
     assert _call_bwd(lib, total_q=0) == 0
     assert _lib.last_error() == ""
