@@ -231,8 +231,8 @@ template <int D, typename E>
 __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   using T = BwdTile<D>;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  // two buffers of a K tile followed by a V tile, filled straight from global memory, in the layout
-  // that serves the reads by rows and the transposing reads (BwdTile::swz_both)
+  // three K tiles and two V tiles, filled straight from global memory, in the layout that serves the reads by
+  // rows and the transposing reads (BwdTile::swz_both)
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -307,15 +307,24 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   int j = -1, kpos = 0;
   int word_base = -32;      // k block of bit 0 of the word being walked
   uint32_t word_left = 0;   // its kept blocks not visited yet
+  // The bit row is read once, a word per lane (64 words = 2048 k blocks at a time), so that no load and its wait
+  // stand between two tiles.
+  const int last_word = (inf.nkblk - 1) >> 5;
+  uint32_t row_words = lane <= last_word ? bits[lane] : 0u;
   auto next_tile = [&]() -> bool {
     if (j >= 0) {
       kpos += kTileKeys;
       if (kpos < min((j + 1) * p.kbs, inf.kmax)) return true;
     }
-    while (word_left == 0) {   // one load per 32 k blocks, kept or not
+    while (word_left == 0) {   // next word of the bit row: 32 k blocks, kept or not
       word_base += 32;
       if (word_base >= inf.nkblk) return false;
-      word_left = bits[word_base >> 5];
+      const int w = word_base >> 5;
+      if (w >= 64 && (w & 63) == 0) {   // beyond 2048 k blocks: the next 64 words, waited for here so that no other path waits
+        row_words = w + lane <= last_word ? bits[w + lane] : 0u;
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+      }
+      word_left = (uint32_t)__builtin_amdgcn_readlane((int)row_words, w & 63);
     }
     j = word_base + __builtin_ctz(word_left);
     word_left &= word_left - 1;
@@ -332,27 +341,28 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   const uint32_t k_s32 = (uint32_t)p.k_s, v_s32 = (uint32_t)p.v_s;              // the host checks that they fit
   const uint32_t k_voff = (uint32_t)ld_row * k_s32 + ld_chunk, v_voff = (uint32_t)ld_row * v_s32 + ld_chunk;   // of a full tile's first load
   const uint32_t tiles_addr = (uint32_t)(uintptr_t)HBSA_AS3(lds) + (uint32_t)wave * 1024u;
-  auto fetch = [&](int buf) {   // the tile next_tile() has just moved to
-    const int valid = tile_valid();
-    const char *ksrc = kg + (int64_t)kpos * p.k_s, *vsrc = vg + (int64_t)kpos * p.v_s;
-    const uint32_t dst = tiles_addr + (uint32_t)(buf * 2 * T::TILE_BYTES);
+  // LDS: three K tiles, then two V tiles.  K tiles are requested two tiles ahead, V tiles one (with two workgroups
+  // of 5 tiles of D = 128 a CU's LDS is full).
+  auto fetch_one = [&](uint32_t dst, const char *src, int64_t stride, uint32_t s32, uint32_t full_voff, int valid) {
     if (valid == kTileKeys) {   // a full tile: the loads differ in their scalar base only
 #pragma unroll
-      for (int i = 0; i < LOADS; ++i) {
-        bwd_dma16(dst + (uint32_t)(i * 4 * 1024), ksrc + (int64_t)(4 * RPL * i) * p.k_s, k_voff);
-        bwd_dma16(dst + (uint32_t)(T::TILE_BYTES + i * 4 * 1024), vsrc + (int64_t)(4 * RPL * i) * p.v_s, v_voff);
-      }
+      for (int i = 0; i < LOADS; ++i) bwd_dma16(dst + (uint32_t)(i * 4 * 1024), src + (int64_t)(4 * RPL * i) * stride, full_voff);
     } else {
 #pragma unroll
       for (int i = 0; i < LOADS; ++i) {
         const uint32_t rr = (uint32_t)min(ld_row + 4 * RPL * i, valid - 1);   // rows past the end repeat the last one (masked later)
-        bwd_dma16(dst + (uint32_t)(i * 4 * 1024), ksrc, rr * k_s32 + ld_chunk);
-        bwd_dma16(dst + (uint32_t)(T::TILE_BYTES + i * 4 * 1024), vsrc, rr * v_s32 + ld_chunk);
+        bwd_dma16(dst + (uint32_t)(i * 4 * 1024), src, rr * s32 + ld_chunk);
       }
     }
   };
-  // Operand addresses of the K tile in use (the V tile lies one tile further, an immediate): they move to the
-  // other buffer with one addition per tile instead of one per read.
+  auto fetch_k = [&](int kb, int at, int valid) {
+    fetch_one(tiles_addr + (uint32_t)(kb * T::TILE_BYTES), kg + (int64_t)at * p.k_s, p.k_s, k_s32, k_voff, valid);
+  };
+  auto fetch_v = [&](int vb, int at, int valid) {
+    fetch_one(tiles_addr + (uint32_t)((3 + vb) * T::TILE_BYTES), vg + (int64_t)at * p.v_s, p.v_s, v_s32, v_voff, valid);
+  };
+  // Operand addresses of the K tile in use: they move to the next buffer with one addition per tile instead of
+  // one per read (the V tile's reads add the distance between the two buffers in use).
   BwdOperandOffsets<D> off;
   off.init(lane);
   {
@@ -366,33 +376,64 @@ __global__ __launch_bounds__(kThreads, 2) void hbsa_bwd_dq_kernel(BwdParams p) {
   // Reads of one half tile's two chains S^T = K Q^T and dP^T = V dO^T: K and V rows in turn, PF under way
   constexpr int PF = 4, NC = 2 * T::KSTEPS;
   static_assert(NC >= PF, "the first reads of a half are issued as one group");
-  bool have = next_tile();
-  int buf = 0;
-  if (have) fetch(0);
-  while (have) {
-    const int cur_kpos = kpos, valid = tile_valid();
-    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the tile has landed
-    __syncthreads();                      // ... every wavefront's, and the other buffer has been read by all
-    const int cur_buf = buf;
-    have = next_tile();
-    if (have) fetch(buf ^ 1);   // on its way while this tile is computed on
-    buf ^= 1;
+  static_assert(LOADS <= 15, "vmcnt immediate");
+  // What was loaded so far (the rows' Q above all, first used in the loop) has arrived before the first tile is
+  // requested: the compiler counts only the loads it knows, and a wait of its own for them inside the loop would
+  // also wait for every tile under way.
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+  bool have_c = next_tile(), have_n = false;   // the current tile exists; the one after it exists (its K is requested)
+  int kpos_c = 0, valid_c = 0, kpos_n = 0, valid_n = 0;
+  int kb = 0, vb = 0;   // K and V buffer of the current tile
+  if (have_c) {
+    kpos_c = kpos;
+    valid_c = tile_valid();
+    fetch_k(0, kpos_c, valid_c);
+    fetch_v(0, kpos_c, valid_c);
+    have_n = next_tile();
+    if (have_n) {
+      kpos_n = kpos;
+      valid_n = tile_valid();
+      fetch_k(1, kpos_n, valid_n);
+    }
+  }
+  while (have_c) {
+    const int cur_kpos = kpos_c, valid = valid_c, cur_kb = kb, cur_vb = vb;
+    // This wavefront's part of the tile has landed; the K loads of the tile after it (requested last; a
+    // wavefront's loads return in order) may still be under way.
+    if (have_n) __builtin_amdgcn_s_waitcnt(0x0F70 | LOADS);   // vmcnt(LOADS)
+    else __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0)
+    __syncthreads();   // ... every wavefront's, and the buffers of the tile before have been read by all
+    if (have_n) fetch_v(vb ^ 1, kpos_n, valid_n);
+    const bool have_nn = have_n && next_tile();
+    kpos_c = kpos_n;
+    valid_c = valid_n;
+    have_c = have_n;
+    if (have_nn) {
+      kpos_n = kpos;
+      valid_n = tile_valid();
+      fetch_k(kb == 0 ? 2 : kb - 1, kpos_n, valid_n);   // two tiles ahead
+    }
+    have_n = have_nn;
+    kb = kb == 2 ? 0 : kb + 1;
+    vb ^= 1;
     if (!active) continue;
-    if (off_buf != cur_buf) {
-      const uint32_t step = (uint32_t)((cur_buf - off_buf) * 2 * T::TILE_BYTES);
+    if (off_buf != cur_kb) {
+      const uint32_t step = (uint32_t)((cur_kb - off_buf) * T::TILE_BYTES);
 #pragma unroll
       for (int ks = 0; ks < T::KSTEPS; ++ks) off.rows[ks] += step;
 #pragma unroll
       for (int dt = 0; dt < T::DT; ++dt) off.tr[dt] += step;
-      off_buf = cur_buf;
+      off_buf = cur_kb;
     }
+    const uint32_t v_from_k = (uint32_t)((3 + cur_vb - cur_kb) * T::TILE_BYTES);   // from a K tile address to the V tile's
     int lim = valid;   // keys of the tile below lim are visible to this lane's row
     if (p.causal) lim = min(lim, lane_kvis - cur_kpos + 1);
     lim -= 4 * g32;
     short8v rb[PF];
     auto chain_read = [&](auto h_, auto i_) {
       constexpr int h = decltype(h_)::value, i = decltype(i_)::value;
-      rb[i % PF] = lds_read_b128<h * 32 * T::RB + (i & 1) * T::TILE_BYTES>(off.rows[i >> 1]);
+      if constexpr (i & 1) rb[i % PF] = lds_read_b128<h * 32 * T::RB>(off.rows[i >> 1] + v_from_k);
+      else rb[i % PF] = lds_read_b128<h * 32 * T::RB>(off.rows[i >> 1]);
     };
     // edge: some key of the tile is hidden from some row of the wavefront (the tile's end, or the causal
     // diagonal); elsewhere the per-element comparison and select are left out.  Rows past the block's end
@@ -761,11 +802,12 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
           continue;
         }
       }
-      while (kept == 0) {   // one load per 64 q blocks: lane i looks at q block kept_base + i
+      while (kept == 0) {   // one load per 64 q blocks: lane i looks at q block kept_base + i; waited for here so that no other path waits
         kept_base += 64;
         if (kept_base >= qb_end) return false;
         uint32_t word = 0;
         if (kept_base + lane < qb_end) word = p.bits[((size_t)hk * p.nqb + kept_base + lane) * p.wpr + (kbl >> 5)];
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         kept = __ballot((word >> (kbl & 31)) & 1u);
       }
       qb = kept_base + __builtin_ctzll(kept);
@@ -1009,8 +1051,8 @@ __global__ __launch_bounds__(512, 1) void hbsa_bwd_dkv8_kernel(BwdParams p) {
 template <int D, typename E>
 int launch_bwd(const BwdParams &bp, int nhead_k, int num_k_block, hipStream_t stream) {
   using T = BwdTile<D>;
-  // LDS: the dQ kernel's two K/V tile pairs; the dK/dV kernels' tile buffers, P records and row values
-  const int lds_dq = 4 * T::TILE_BYTES, lds_dkv = D == 128 ? 9 * T::TILE_BYTES + 2048 : 4 * T::TILE_BYTES + 1024;
+  // LDS: the dQ kernel's three K and two V tiles; the dK/dV kernels' tile buffers, P records and row values
+  const int lds_dq = 5 * T::TILE_BYTES, lds_dkv = D == 128 ? 9 * T::TILE_BYTES + 2048 : 4 * T::TILE_BYTES + 1024;
   if (lds_dkv > 48 * 1024) {
     static thread_local bool raised[kMaxDevices] = {};
     int dev = 0;
