@@ -322,7 +322,7 @@ int hbsa_fwd_run_lse(const void *q, const void *k, const void *v, void *out,
  * (bf16 keeps fp32's range), with out and lse from a forward on those copies, and widens the gradients, which
  * is what the Python operator does.
  * Head dims above 128 are refused: the dK/dV kernel keeps K^T or V^T of a wavefront's keys and one accumulator
- * in registers, 241 of 256 at headdim 128.
+ * in registers, 254 of 256 at headdim 128.
  */
 size_t hbsa_bwd_workspace_bytes(int32_t total_q, int32_t nhead_q);
 
