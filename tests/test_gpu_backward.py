@@ -70,6 +70,14 @@ CASES = [
     (10, [513], [1029], 2, 2, 128, 64, 192, 0.5, False, None),
     (11, [200, 150], [180, 260], 16, 8, 64, 64, 64, 0.5, True, None),     # eight kv heads: the grid decoded by XCD
     (12, [300], [300], 16, 16, 128, 128, 128, 0.6, True, None),
+    # more than 64 q blocks in a sequence (the dK/dV kernels look at them 64 at a time), many tiles per workgroup
+    # (tiles are fetched two ahead), a ragged last block
+    (13, [9000, 700], [9000, 450], 2, 2, 128, 128, 128, 0.15, True, None),
+    (14, [8500], [8200], 2, 1, 64, 64, 128, 0.2, True, None),
+    # more than 2048 k blocks in a sequence (the dQ kernel holds 64 words of its bit row at a time), 16-key blocks
+    # (half-empty wave slots in the dK/dV kernels)
+    (15, [200], [35000], 2, 1, 128, 64, 16, 0.05, False, None),
+    (16, [150, 40], [33000, 100], 2, 2, 64, 32, 16, 0.05, True, None),
 ]
 
 
