@@ -66,7 +66,7 @@ struct BwdTile {
   // bits select the 64-byte column group.  Over any 16 consecutive rows the 16-byte slots of a chunk
   // column are all different (reads by rows), and rows 0-7 of a group spread evenly over the column
   // groups (transposing reads).
-  static __device__ __forceinline__ int swz_both(int r) {
+  static __host__ __device__ constexpr int swz_both(int r) {
     const int a = (r / RPG) % CPR;
     if constexpr (CPR == 16) return ((a & 3) << 2) | (a >> 2);
     else if constexpr (CPR == 8) return ((a & 1) << 2) | (a >> 1);
@@ -97,6 +97,12 @@ template <int D>
 struct BwdOperandOffsets {
   using T = BwdTile<D>;
   uint32_t rows[T::KSTEPS], tr[T::DT];
+  static constexpr bool second_read_is_xor_32() {
+    for (int key = 0; key < 8; ++key)
+      if (T::swz_both(key + 8) != (T::swz_both(key) ^ 2)) return false;
+    return true;
+  }
+  static_assert(second_read_is_xor_32(), "the second transposing read's address is derived from the first one's");
   __device__ __forceinline__ void init(int lane) {
     const int l32 = lane & 31, g32 = lane >> 5;
     const int rd = l32 * T::RB + ((g32 ^ T::swz_both(l32)) << 4);
