@@ -128,7 +128,7 @@ struct FwdParams {
   int32_t f32;    // fp32 inputs staged as fp16: the softmax constants come from the launch record, where
                   // the setup kernel derived them from the tensors' maxima
   int32_t nhead_k;
-  int32_t one_each;   // > 0: the number of work items, handed out without queues: workgroup i takes items i, i + grid, ...
+  int32_t one_each;   // > 0: the number of work items, handed out without the per-XCD queues: workgroup i takes item i, then items from one counter
   struct Sched *sched;
   // Walk order of the kept k blocks (see the kernel's comment).  walk != 0: the workgroups that work on
   // one (kv head, sequence) keep near each other in key space through a shared clock, so that they find
@@ -153,6 +153,7 @@ struct FwdParams {
   int64_t ms_h, ms_q;                             // its head and q block strides
   int32_t batch, nkb_total, total_k, qbs;
   int32_t pack;   // host side only: the launch uses the kernel whose wave slots are packed across the q heads of a GQA group
+  FastDiv div_nhk;   // division by nhead_k (items handed out without queues)
 };
 
 // Boundaries of one sequence of the packed batch, as read from the caller's device arrays.
@@ -406,10 +407,11 @@ __global__ __launch_bounds__(256) void hbsa_f32_stage_kernel(F32Tensor t, const 
 }
 
 constexpr int kListCap = 1024;   // tile entries per list; longer items are expanded in chunks
-// Up to this many items per resident workgroup are dealt out in turn, without the work queues (measured: 8 x 512
-// tokens 71 -> 48 us, 8 x 1024 113 -> 106, C5 0.33 -> 0.28 ms; at eight per workgroup a causal mask's uneven items cost
-// more than the queues do: 8 x 2048 causal 204 -> 247 us).
-constexpr int kStaticShare = 4;
+// Up to this many items per resident workgroup are handed out without the per-XCD work queues: two fixed items per
+// workgroup, the rest from one counter (see claim() in the kernel).  Measured against the queues: 8 x 512 tokens
+// 71 -> 45 us, 8 x 1024 113 -> 105, 8 x 2048 causal 200 -> 190, C5 0.33 -> 0.255 ms; at sixteen per workgroup 8 x 4096
+// tokens lose 1 % (the queues keep one head's K/V in one XCD's L2).
+constexpr int kStaticShare = 8;
 // One-launch form: sequences whose boundaries the scheduler keeps in LDS (batch + 1 entries of four arrays),
 // and bytes of its staging area for one row of block_mask bytes (2048 blocks and the alignment slack)
 constexpr int kSeqCap = 128;
@@ -614,7 +616,7 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
   // counts the workgroup as done, and the workgroup that completes the count puts the queue counters
   // back to zero, so the next launch on this work description needs no preparation of its own.
   auto leave = [&]() {
-    if (wave != 0 || p.one_each) return;
+    if (wave != 0 || (p.one_each && (uint32_t)p.one_each <= 2u * gridDim.x)) return;   // (at most two fixed items per workgroup: no counter was touched)
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this workgroup's last claim has returned
     if (lane == 0) {
       const uint32_t before = atomicAdd(&p.sched->done, 1u);
@@ -639,12 +641,22 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
     const int heads = v < p.nhead_k ? (p.nhead_k - v + 7) / 8 : 0;
     return (uint32_t)heads * (uint32_t)p.nqb * (uint32_t)p.nsub * (uint32_t)p.nparts;
   };
-  uint32_t own_next = blockIdx.x;   // one_each: this workgroup's next item
+  // Without queues (few items per workgroup).  The items are numbered last q blocks first, the heads of a q block
+  // next to each other (decode_free_entry), so under a causal mask their weights fall with the number.  Workgroup
+  // i of G takes item i, then item 2G - 1 - i (the lightest second item goes to the heaviest first one), and
+  // what lies beyond 2G is claimed from one counter as workgroups become free: uneven items (a causal mask,
+  // ragged sequences) then do not leave the workgroups, and the workgroups of one CU, with uneven sums.  Both
+  // fixed items are known at once, so no claim's latency is waited for before the first tile.
+  int own_claims = 0;
+  bool counter_dry = false;   // a claim from the counter has come back past the last item
   auto claim = [&]() -> uint32_t {   // the value is looked at an item later, so its latency is hidden
     uint32_t r = 0xffffffffu;
     if (p.one_each) {
-      if (own_next < (uint32_t)p.one_each) r = own_next;
-      own_next += gridDim.x;
+      if (own_claims == 0) r = blockIdx.x;
+      else if (own_claims == 1) r = 2u * gridDim.x - 1u - blockIdx.x;
+      else if ((uint32_t)p.one_each > 2u * gridDim.x && !counter_dry && lane == 0)
+        r = 2u * gridDim.x + atomicAdd(&p.sched->qnext[0], 1u);
+      ++own_claims;
     } else if (tries < 8) {
       if (lane == 0) r = atomicAdd(&p.sched->qnext[(first_queue + tries) & 7], 1u);
     }
@@ -660,6 +672,17 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
     const uint32_t h = fast_div(t, p.div_nqb);
     st_hk = head0 + head_step * (int)h;
     st_qb = p.nqb - 1 - (int)(t - h * (uint32_t)p.nqb);
+  };
+  // (kv head, q block, slot group, part) of item `claimed` of the numbering without queues: parts, slot groups and
+  // kv heads of a q block are neighbours, the last q block comes first
+  auto decode_free_entry = [&](uint32_t claimed) {
+    const uint32_t whole = fast_div(claimed, p.div_nparts);
+    st_part = (int)(claimed - whole * (uint32_t)p.nparts);
+    const uint32_t t = fast_div(whole, p.div_nsub);
+    st_sub = (int)(whole - t * (uint32_t)p.nsub);
+    const uint32_t b = fast_div(t, p.div_nhk);
+    st_hk = (int)(t - b * (uint32_t)p.nhead_k);
+    st_qb = p.nqb - 1 - (int)b;
   };
   // ---- one-launch form: geometry and mask bits without a pre-pass (wavefront 0)
   const uint8_t *st_mrow = nullptr;   // staged item: address of the mask byte of its sequence's first k block
@@ -749,7 +772,8 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
     uint32_t claimed = (uint32_t)__builtin_amdgcn_readfirstlane((int)pending);
     st_hk = -1;
     if (p.one_each) {
-      if (claimed != 0xffffffffu) decode_entry(claimed, 0, 1);
+      if (claimed < (uint32_t)p.one_each) decode_free_entry(claimed);
+      else if (own_claims > 2) counter_dry = true;
     } else {
       while (tries < 8) {
         const int v = (first_queue + tries) & 7;
@@ -1746,6 +1770,7 @@ void fill_shape(FwdParams &fp, int nhead_q, int nhead_k, int headdim, int num_q_
   fp.nsub = (slots + fp.nw - 1) / fp.nw;
   fp.div_nsub = make_fast_div((uint32_t)fp.nsub);
   fp.div_nqb = make_fast_div((uint32_t)num_q_block);
+  fp.div_nhk = make_fast_div((uint32_t)nhead_k);
   fp.div_kbs = make_fast_div((uint32_t)k_block_size);
   fp.q_sign = softmax_scale < 0.f ? 0x80008000u : 0u;
   float c = std::fabs(softmax_scale) * kLog2e;
@@ -1772,8 +1797,8 @@ int launch_fwd_nw(const FwdParams &fp, long long items, hipStream_t stream) {
   }
   const int grid = (int)(items < resident ? items : resident);
   FwdParams launch = fp;
-  // Few items per workgroup: they are dealt out in turn (heaviest first, so the shares are even), without queues
-  // or atomics, whose round trips would be a good part of such a launch.
+  // Few items per workgroup: two fixed ones each and one counter for the rest instead of the per-XCD queues, whose
+  // round trips (and, with few kv heads, the crowd at few counters) would be a good part of such a launch.
   launch.one_each = items <= (long long)kStaticShare * resident ? (int)items : 0;
   hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS, FUSED, PACK>), dim3(grid), dim3(NW * 64), lds_bytes, stream, launch);
   hipError_t e = hipGetLastError();
