@@ -128,7 +128,7 @@ struct FwdParams {
   int32_t f32;    // fp32 inputs staged as fp16: the softmax constants come from the launch record, where
                   // the setup kernel derived them from the tensors' maxima
   int32_t nhead_k;
-  int32_t one_each;   // > 0: the number of work items, handed out without the per-XCD queues: workgroup i takes item i, then items from one counter
+  int32_t one_each;   // > 0: the number of work items, handed out without queues: workgroup i of G takes items i, 2G - 1 - i, 2G + i, ...
   struct Sched *sched;
   // Walk order of the kept k blocks (see the kernel's comment).  walk != 0: the workgroups that work on
   // one (kv head, sequence) keep near each other in key space through a shared clock, so that they find
@@ -407,10 +407,10 @@ __global__ __launch_bounds__(256) void hbsa_f32_stage_kernel(F32Tensor t, const 
 }
 
 constexpr int kListCap = 1024;   // tile entries per list; longer items are expanded in chunks
-// Up to this many items per resident workgroup are handed out without the per-XCD work queues: two fixed items per
-// workgroup, the rest from one counter (see claim() in the kernel).  Measured against the queues: 8 x 512 tokens
-// 71 -> 45 us, 8 x 1024 113 -> 105, 8 x 2048 causal 200 -> 190, C5 0.33 -> 0.255 ms; at sixteen per workgroup 8 x 4096
-// tokens lose 1 % (the queues keep one head's K/V in one XCD's L2).
+// Up to this many items per resident workgroup are handed out without the per-XCD work queues, in a fixed order
+// (see claim() in the kernel).  Measured against the queues: 8 x 512 tokens 71 -> 45 us, 8 x 1024 113 -> 99,
+// 8 x 2048 causal 200 -> 189, C5 0.33 -> 0.245 ms; at sixteen per workgroup 8 x 4096 tokens lose 5 % and at 64
+// C2 and C3 lose 5-8 % (the queues keep one head's K/V in one XCD's L2).
 constexpr int kStaticShare = 8;
 // One-launch form: sequences whose boundaries the scheduler keeps in LDS (batch + 1 entries of four arrays),
 // and bytes of its staging area for one row of block_mask bytes (2048 blocks and the alignment slack)
@@ -616,7 +616,7 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
   // counts the workgroup as done, and the workgroup that completes the count puts the queue counters
   // back to zero, so the next launch on this work description needs no preparation of its own.
   auto leave = [&]() {
-    if (wave != 0 || (p.one_each && (uint32_t)p.one_each <= 2u * gridDim.x)) return;   // (at most two fixed items per workgroup: no counter was touched)
+    if (wave != 0 || p.one_each) return;   // (items without queues: no counter was touched)
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this workgroup's last claim has returned
     if (lane == 0) {
       const uint32_t before = atomicAdd(&p.sched->done, 1u);
@@ -643,19 +643,15 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
   };
   // Without queues (few items per workgroup).  The items are numbered last q blocks first, the heads of a q block
   // next to each other (decode_free_entry), so under a causal mask their weights fall with the number.  Workgroup
-  // i of G takes item i, then item 2G - 1 - i (the lightest second item goes to the heaviest first one), and
-  // what lies beyond 2G is claimed from one counter as workgroups become free: uneven items (a causal mask,
-  // ragged sequences) then do not leave the workgroups, and the workgroups of one CU, with uneven sums.  Both
-  // fixed items are known at once, so no claim's latency is waited for before the first tile.
+  // i of G takes item i, then 2G - 1 - i, 2G + i, 4G - 1 - i, ...: every second round runs backwards, so the
+  // lightest item of a round goes to the workgroup that got the heaviest of the round before, and the
+  // workgroups (those of one CU, too) end at about the same time.  Nothing is claimed: measured against a shared
+  // counter for the later rounds, 8 x 1024 tokens 106 -> 99 us and C5 0.258 -> 0.241 ms.
   int own_claims = 0;
-  bool counter_dry = false;   // a claim from the counter has come back past the last item
   auto claim = [&]() -> uint32_t {   // the value is looked at an item later, so its latency is hidden
     uint32_t r = 0xffffffffu;
     if (p.one_each) {
-      if (own_claims == 0) r = blockIdx.x;
-      else if (own_claims == 1) r = 2u * gridDim.x - 1u - blockIdx.x;
-      else if ((uint32_t)p.one_each > 2u * gridDim.x && !counter_dry && lane == 0)
-        r = 2u * gridDim.x + atomicAdd(&p.sched->qnext[0], 1u);
+      r = (own_claims & 1) ? (uint32_t)(own_claims + 1) * gridDim.x - 1u - blockIdx.x : (uint32_t)own_claims * gridDim.x + blockIdx.x;
       ++own_claims;
     } else if (tries < 8) {
       if (lane == 0) r = atomicAdd(&p.sched->qnext[(first_queue + tries) & 7], 1u);
@@ -773,7 +769,6 @@ __global__ __launch_bounds__(NW * 64, D > 128 ? 1 : 8 / NW) void hbsa_fwd_kernel
     st_hk = -1;
     if (p.one_each) {
       if (claimed < (uint32_t)p.one_each) decode_free_entry(claimed);
-      else if (own_claims > 2) counter_dry = true;
     } else {
       while (tries < 8) {
         const int v = (first_queue + tries) & 7;
@@ -1797,8 +1792,8 @@ int launch_fwd_nw(const FwdParams &fp, long long items, hipStream_t stream) {
   }
   const int grid = (int)(items < resident ? items : resident);
   FwdParams launch = fp;
-  // Few items per workgroup: two fixed ones each and one counter for the rest instead of the per-XCD queues, whose
-  // round trips (and, with few kv heads, the crowd at few counters) would be a good part of such a launch.
+  // Few items per workgroup: a fixed order instead of the per-XCD queues, whose round trips (and, with few kv
+  // heads, the crowd at few counters) would be a good part of such a launch.
   launch.one_each = items <= (long long)kStaticShare * resident ? (int)items : 0;
   hipLaunchKernelGGL((hbsa_fwd_kernel<D, E, OUT32, NW, EXTRAS, FUSED, PACK>), dim3(grid), dim3(NW * 64), lds_bytes, stream, launch);
   hipError_t e = hipGetLastError();
