@@ -825,6 +825,32 @@ def test_seeded_random_shapes_that_fill_the_device_as_one_launch_and_as_two():
     assert ones >= 20
 
 
+@pytest.mark.parametrize("causal", [True, False], ids=["causal", "full"])
+@pytest.mark.parametrize("seq_len", [256, 384, 640, 1152, 2048, 2176])
+def test_item_counts_around_the_limits_of_the_queue_free_order(seq_len, causal):
+    """8 sequences x 32 heads of 128-row q blocks give 512 to 4352 (kv head, q block) items: one per resident
+    workgroup, a partial second round, a partial third round (the rounds run forwards and backwards in turn), exactly
+    eight rounds, and one more q block per sequence, which goes through the per-XCD queues.  Every item must be
+    worked on exactly once: rows of the first, middle and last q blocks of every sequence against the oracle, and
+    the whole output bit for bit against the two-launch form."""
+    from hbsattn_amd import set_onepass
+    w = make_problem(seed=4242 + seq_len, q_lens=[seq_len] * 8, k_lens=[seq_len] * 8, hq=32, hk=32, d=128, qbs=128, kbs=128,
+                     keep=0.3, diag=True, causal=causal, scale=None)
+    what = f"8 x {seq_len} tokens, causal={causal}"
+    assert _launches(w) == 1, what
+    out = _run(w)
+    rows = []
+    for b in range(8):
+        rows += [b * seq_len, b * seq_len + 127, b * seq_len + seq_len // 2, (b + 1) * seq_len - 128, (b + 1) * seq_len - 1]
+    assert_close_to_oracle(out, oracle_for(w, q_rows=sorted(set(rows))), what)
+    assert torch.isfinite(out.float()).all(), what
+    previous = set_onepass(False)
+    try:
+        assert torch.equal(_run(w), out), what
+    finally:
+        set_onepass(previous)
+
+
 # ---------------------------------------------------------------------------------------
 # head dims above 128 (the reference pads any head dim to a power of two: fwd_triton_auto_tile_size.py:269)
 # ---------------------------------------------------------------------------------------
